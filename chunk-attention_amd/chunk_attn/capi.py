@@ -1,0 +1,473 @@
+"""ctypes binding of libchunkattn_hip.so (the C-ABI declared in include/chunk_attn_hip.h).
+
+`Tree` wraps the prefix-tree manager handle, `KernelContext` the device-side context, and
+`Attention` composes both over a torch-allocated fp16 KV pool with the same methods as the
+pybind11 class (add_seq / append_token / forward / remove_seq / reserve /
+refresh_kernel_context), for hosts that cannot load the C++ extension module.
+
+There is no CPU fallback: loading fails if the library has not been built, and every device
+entry point reports an error when no HIP device is present.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libchunkattn_hip.so")
+_lib = None
+
+c_int_p = ctypes.POINTER(ctypes.c_int)
+c_i32_p = ctypes.POINTER(ctypes.c_int32)
+c_f32_p = ctypes.POINTER(ctypes.c_float)
+
+
+class ChunkRow(ctypes.Structure):
+    _fields_ = [("slot", ctypes.c_int32), ("n_tokens", ctypes.c_int32),
+                ("seq_begin", ctypes.c_int32), ("seq_end", ctypes.c_int32)]
+
+
+class PlanInfo(ctypes.Structure):
+    _fields_ = [("n_seqs", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
+                ("n_shared_chunks", ctypes.c_int32), ("ref_partial_rows", ctypes.c_int32),
+                ("max_seq_n_chunks", ctypes.c_int32), ("n_shared_items", ctypes.c_int32),
+                ("n_stream_items", ctypes.c_int32), ("n_part_rows", ctypes.c_int32),
+                ("shared_tokens", ctypes.c_int64), ("stream_tokens", ctypes.c_int64)]
+
+
+# name -> (restype, argtypes); every symbol include/chunk_attn_hip.h declares
+SIGNATURES = {
+    "ca_last_error": (ctypes.c_char_p, []),
+    "ca_ctx_create": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int,
+                                     ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                     ctypes.c_int]),
+    "ca_ctx_destroy": (None, [ctypes.c_void_p]),
+    "ca_refresh_kernel_context": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ChunkRow),
+                                                 ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "ca_ctx_valid": (ctypes.c_int, [ctypes.c_void_p]),
+    "ca_ctx_invalidate": (None, [ctypes.c_void_p]),
+    "ca_ctx_delta_tokens": (ctypes.c_int, [ctypes.c_void_p]),
+    "ca_ctx_set_delta_tokens": (None, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_attention": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                    ctypes.c_int, ctypes.c_void_p]),
+    "ca_attn_chunks_first": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                            ctypes.c_void_p]),
+    "ca_attn_seqs_first": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_int, ctypes.c_void_p]),
+    "ca_append_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                    ctypes.c_void_p]),
+    "ca_scatter_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                     ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
+    "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
+    "ca_ctx_plan_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
+    "ca_ctx_ref_tables": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
+    "ca_ctx_export_partials": (ctypes.c_int, [ctypes.c_void_p, c_f32_p, c_f32_p, c_f32_p,
+                                              ctypes.c_void_p]),
+    "ca_tables_build": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ChunkRow)] +
+                        [ctypes.c_int] * 9),
+    "ca_tables_destroy": (None, [ctypes.c_void_p]),
+    "ca_tables_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
+    "ca_tables_plan_sizes": (ctypes.c_int, [ctypes.c_void_p, c_int_p, c_int_p]),
+    "ca_tables_ref": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
+    "ca_tables_plan": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 8),
+    "ca_tree_create": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_int]),
+    "ca_tree_destroy": (None, [ctypes.c_void_p]),
+    "ca_tree_max_chunks_for": (ctypes.c_int, [ctypes.c_int] * 5),
+    "ca_tree_add_seq": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p, c_int_p,
+                                       c_i32_p, ctypes.c_int, c_int_p]),
+    "ca_tree_remove_seq": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_tree_clear": (ctypes.c_int, [ctypes.c_void_p]),
+    "ca_tree_reserve": (ctypes.c_int, [ctypes.c_void_p, c_int_p]),
+    "ca_tree_append_token": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p]),
+    "ca_tree_get_chunks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ChunkRow), ctypes.c_int,
+                                          c_int_p]),
+    "ca_tree_n_seqs": (ctypes.c_int, [ctypes.c_void_p]),
+    "ca_tree_used_chunks": (ctypes.c_int, [ctypes.c_void_p]),
+    "ca_tree_version": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "ca_tree_tails": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p]),
+    "ca_tree_dump": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p, c_i32_p,
+                                    ctypes.c_int, c_int_p]),
+}
+
+
+def load() -> ctypes.CDLL:
+    """The C-ABI library, with argument types set.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(
+                f"{_LIB_PATH} is missing: build it with `python chunk-attention_amd/build.py` "
+                "(the decode path has no fallback implementation)")
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class ChunkAttnError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(message)
+        self.code = code
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise ChunkAttnError(rc, load().ca_last_error().decode())
+
+
+def _i32(values: Sequence[int]):
+    arr = np.ascontiguousarray(np.asarray(values, dtype=np.int32))
+    return arr, arr.ctypes.data_as(c_i32_p)
+
+
+class Tree:
+    """Prefix-tree chunk manager handle (ca_tree_*)."""
+
+    def __init__(self, chunk_size: int, max_chunks: int, share_prefix: bool = True):
+        self._lib = load()
+        self._h = ctypes.c_void_p()
+        _check(self._lib.ca_tree_create(ctypes.byref(self._h), chunk_size, max_chunks, int(share_prefix)))
+        self.chunk_size = chunk_size
+        self.max_chunks = max_chunks
+
+    def __del__(self):
+        if getattr(self, "_h", None) and self._h.value:
+            self._lib.ca_tree_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def add_seq(self, tokens: Sequence[int]) -> Tuple[int, int, List[int]]:
+        """Returns (seq_idx, tok_begin, slots): tokens[tok_begin:] need their K/V copied into
+        `slots`, chunk_size rows each."""
+        arr, ptr = _i32(tokens)
+        cap = len(tokens) // self.chunk_size + 2
+        slots = (ctypes.c_int32 * cap)()
+        idx, tb, n_new = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _check(self._lib.ca_tree_add_seq(self._h, ptr, len(tokens), ctypes.byref(idx), ctypes.byref(tb),
+                                         slots, cap, ctypes.byref(n_new)))
+        return idx.value, tb.value, list(slots[: n_new.value])
+
+    def remove_seq(self, seq_idx: int) -> None:
+        _check(self._lib.ca_tree_remove_seq(self._h, seq_idx))
+
+    def clear(self) -> None:
+        _check(self._lib.ca_tree_clear(self._h))
+
+    def reserve(self) -> int:
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_reserve(self._h, ctypes.byref(n)))
+        return n.value
+
+    def append_token(self, tokens: Sequence[int]) -> int:
+        arr, ptr = _i32(tokens)
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_append_token(self._h, ptr, len(tokens), ctypes.byref(n)))
+        return n.value
+
+    def get_chunks(self) -> np.ndarray:
+        """[n_rows, 4] int32: slot, n_tokens, seq_begin, seq_end in get_chunks order."""
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_get_chunks(self._h, None, 0, ctypes.byref(n)))
+        rows = np.zeros((max(n.value, 1), 4), np.int32)
+        _check(self._lib.ca_tree_get_chunks(self._h, rows.ctypes.data_as(ctypes.POINTER(ChunkRow)),
+                                            n.value, ctypes.byref(n)))
+        return rows[: n.value]
+
+    @property
+    def n_seqs(self) -> int:
+        return self._lib.ca_tree_n_seqs(self._h)
+
+    @property
+    def used_chunks(self) -> int:
+        return self._lib.ca_tree_used_chunks(self._h)
+
+    @property
+    def version(self) -> int:
+        return self._lib.ca_tree_version(self._h)
+
+    def tails(self) -> List[int]:
+        n = ctypes.c_int()
+        cap = max(self.n_seqs, 1)
+        buf = (ctypes.c_int32 * cap)()
+        _check(self._lib.ca_tree_tails(self._h, buf, cap, ctypes.byref(n)))
+        return list(buf[: n.value])
+
+    def dump(self):
+        """Pre-order list of (depth, n_seqs, tokens, slot), children first-to-last."""
+        nn, nt = ctypes.c_int(), ctypes.c_int()
+        _check(self._lib.ca_tree_dump(self._h, None, 0, ctypes.byref(nn), None, 0, ctypes.byref(nt)))
+        nodes = np.zeros((max(nn.value, 1), 4), np.int32)
+        toks = np.zeros(max(nt.value, 1), np.int32)
+        _check(self._lib.ca_tree_dump(self._h, nodes.ctypes.data_as(c_i32_p), nn.value, ctypes.byref(nn),
+                                      toks.ctypes.data_as(c_i32_p), nt.value, ctypes.byref(nt)))
+        out, pos = [], 0
+        for depth, n_seqs, n_tok, slot in nodes[: nn.value].tolist():
+            out.append((depth, n_seqs, toks[pos: pos + n_tok].tolist(), slot))
+            pos += n_tok
+        return out
+
+    def structure(self):
+        """Nested (n_seqs, tokens, [children]) like the oracle's PrefixTree.structure()."""
+        flat = self.dump()
+        root = (flat[0][1], tuple(flat[0][2]), [])
+        stack = [(0, root)]
+        for depth, n_seqs, toks, _ in flat[1:]:
+            node = (n_seqs, tuple(toks), [])
+            while stack[-1][0] >= depth:
+                stack.pop()
+            stack[-1][1][2].append(node)
+            stack.append((depth, node))
+        return root
+
+
+def max_chunks_for(memory_mb: int, chunk_size: int, n_heads: int, d_head: int, elem_bytes: int = 2) -> int:
+    return load().ca_tree_max_chunks_for(memory_mb, chunk_size, n_heads, d_head, elem_bytes)
+
+
+def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: int = 1,
+                 partition: int = 0, shared_seg_chunks: int = 0, stream_chunks: int = 0,
+                 n_heads: int = 32, n_cus: int = 256) -> dict:
+    """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
+    (work items as [n, 8] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
+    len_seq, reserved)."""
+    lib = load()
+    rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
+    h = ctypes.c_void_p()
+    _check(lib.ca_tables_build(ctypes.byref(h), rows.ctypes.data_as(ctypes.POINTER(ChunkRow)),
+                               rows.shape[0], n_seqs, chunk_size, tpp_threshold, partition,
+                               shared_seg_chunks, stream_chunks, n_heads, n_cus))
+    try:
+        info = PlanInfo()
+        _check(lib.ca_tables_info(h, ctypes.byref(info)))
+        n_slots, n_list = ctypes.c_int(), ctypes.c_int()
+        _check(lib.ca_tables_plan_sizes(h, ctypes.byref(n_slots), ctypes.byref(n_list)))
+        t = {
+            "final_idx": np.zeros(info.n_chunks, np.int32),
+            "slots": np.zeros(info.n_chunks, np.int32),
+            "begins": np.zeros(info.n_shared_chunks, np.int32),
+            "ends": np.zeros(info.n_shared_chunks, np.int32),
+            "offsets": np.zeros(info.n_shared_chunks, np.int32),
+            "seq_n_tokens": np.zeros(info.n_seqs, np.int32),
+            "seq_chunk_map": np.zeros((info.n_seqs, info.max_seq_n_chunks), np.int32),
+        }
+        _check(lib.ca_tables_ref(h, *[t[k].ctypes.data_as(c_i32_p) for k in (
+            "final_idx", "slots", "begins", "ends", "offsets", "seq_n_tokens", "seq_chunk_map")]))
+        t["n_shared"] = info.n_shared_chunks
+        t["partial_rows"] = info.ref_partial_rows
+        t["max_seq_n_chunks"] = info.max_seq_n_chunks
+        p = {
+            "shared_items": np.zeros((info.n_shared_items, 8), np.int32),
+            "stream_items": np.zeros((info.n_stream_items, 8), np.int32),
+            "slots": np.zeros(n_slots.value, np.int32),
+            "seq_len": np.zeros(info.n_seqs, np.int32),
+            "part_ptr": np.zeros(info.n_seqs + 1, np.int32),
+            "part_rows": np.zeros(n_list.value, np.int32),
+            "tail_slot": np.zeros(info.n_seqs, np.int32),
+            "tail_fill": np.zeros(info.n_seqs, np.int32),
+        }
+        _check(lib.ca_tables_plan(h, *[p[k].ctypes.data_as(c_i32_p) for k in (
+            "shared_items", "stream_items", "slots", "seq_len", "part_ptr", "part_rows",
+            "tail_slot", "tail_fill")]))
+        p["n_part_rows"] = info.n_part_rows
+        p["shared_tokens"] = info.shared_tokens
+        p["stream_tokens"] = info.stream_tokens
+        return {"ref": t, "plan": p}
+    finally:
+        lib.ca_tables_destroy(h)
+
+
+class KernelContext:
+    """Device-side context handle (ca_ctx_*).  Pointers are raw device addresses."""
+
+    def __init__(self, n_heads: int, d_head: int, chunk_size: int, k_pool_ptr: int, v_pool_ptr: int,
+                 max_chunks: int, tpp_threshold: int = 1):
+        self._lib = load()
+        self._h = ctypes.c_void_p()
+        _check(self._lib.ca_ctx_create(ctypes.byref(self._h), n_heads, d_head, chunk_size, k_pool_ptr,
+                                       v_pool_ptr, max_chunks, tpp_threshold))
+        self.n_heads, self.d_head, self.chunk_size = n_heads, d_head, chunk_size
+
+    def __del__(self):
+        if getattr(self, "_h", None) and self._h.value:
+            self._lib.ca_ctx_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def refresh(self, rows: np.ndarray, n_seqs: int, stream: int = 0) -> None:
+        rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
+        _check(self._lib.ca_refresh_kernel_context(
+            self._h, rows.ctypes.data_as(ctypes.POINTER(ChunkRow)), rows.shape[0], n_seqs, stream))
+
+    @property
+    def valid(self) -> bool:
+        return bool(self._lib.ca_ctx_valid(self._h))
+
+    def invalidate(self) -> None:
+        self._lib.ca_ctx_invalidate(self._h)
+
+    @property
+    def delta_tokens(self) -> int:
+        return self._lib.ca_ctx_delta_tokens(self._h)
+
+    @delta_tokens.setter
+    def delta_tokens(self, v: int) -> None:
+        self._lib.ca_ctx_set_delta_tokens(self._h, v)
+
+    def attention(self, q_ptr: int, out_ptr: int, n_seqs: int, partition: int = 0, stream: int = 0) -> None:
+        _check(self._lib.ca_attention(self._h, q_ptr, out_ptr, n_seqs, partition, stream))
+
+    def attn_chunks_first(self, q_ptr: int, n_seqs: int, stream: int = 0) -> None:
+        _check(self._lib.ca_attn_chunks_first(self._h, q_ptr, n_seqs, stream))
+
+    def attn_seqs_first(self, q_ptr: int, out_ptr: int, n_seqs: int, stream: int = 0) -> None:
+        _check(self._lib.ca_attn_seqs_first(self._h, q_ptr, out_ptr, n_seqs, stream))
+
+    def append_kv(self, k_ptr: int, v_ptr: int, n_seqs: int, stream: int = 0) -> None:
+        _check(self._lib.ca_append_kv(self._h, k_ptr, v_ptr, n_seqs, stream))
+
+    def scatter_kv(self, k_ptr: int, v_ptr: int, n_tokens: int, tok_begin: int, slots: Sequence[int],
+                   stream: int = 0) -> None:
+        arr, ptr = _i32(slots)
+        _check(self._lib.ca_scatter_kv(self._h, k_ptr, v_ptr, n_tokens, tok_begin, ptr, len(slots), stream))
+
+    def copy_chunk(self, src_slot: int, dst_slot: int, stream: int = 0) -> None:
+        _check(self._lib.ca_copy_chunk(self._h, src_slot, dst_slot, stream))
+
+    def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
+        _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
+
+    def plan_info(self) -> PlanInfo:
+        info = PlanInfo()
+        _check(self._lib.ca_ctx_plan_info(self._h, ctypes.byref(info)))
+        return info
+
+    def ref_tables(self) -> dict:
+        info = self.plan_info()
+        t = {
+            "final_idx": np.zeros(info.n_chunks, np.int32),
+            "slots": np.zeros(info.n_chunks, np.int32),
+            "begins": np.zeros(info.n_shared_chunks, np.int32),
+            "ends": np.zeros(info.n_shared_chunks, np.int32),
+            "offsets": np.zeros(info.n_shared_chunks, np.int32),
+            "seq_n_tokens": np.zeros(info.n_seqs, np.int32),
+            "seq_chunk_map": np.zeros((info.n_seqs, info.max_seq_n_chunks), np.int32),
+        }
+        _check(self._lib.ca_ctx_ref_tables(self._h, *[t[k].ctypes.data_as(c_i32_p) for k in (
+            "final_idx", "slots", "begins", "ends", "offsets", "seq_n_tokens", "seq_chunk_map")]))
+        t["n_shared"] = info.n_shared_chunks
+        t["partial_rows"] = info.ref_partial_rows
+        return t
+
+    def export_partials(self, stream: int = 0):
+        """(maxs, sums [rows*H], attns [rows*H, d]) in the reference's partial layout."""
+        info = self.plan_info()
+        n = info.ref_partial_rows * self.n_heads
+        maxs = np.zeros(n, np.float32)
+        sums = np.zeros(n, np.float32)
+        attns = np.zeros((n, self.d_head), np.float32)
+        _check(self._lib.ca_ctx_export_partials(self._h, maxs.ctypes.data_as(c_f32_p),
+                                                sums.ctypes.data_as(c_f32_p),
+                                                attns.ctypes.data_as(c_f32_p), stream))
+        return maxs, sums, attns
+
+
+class Attention:
+    """Prefix-tree KV cache + decode attention over the C-ABI, torch tensors in and out.
+
+    Same methods and argument meaning as the pybind11 `Attention` class; chunks are reported
+    as pool slot ids instead of node objects."""
+
+    def __init__(self, n_heads: int = 12, d_head: int = 64, chunk_size: int = 64, memory_mb: int = 1024,
+                 share_prefix: bool = True, tpp_threshold: int = 1, dtype=None, device=None):
+        import torch
+        dtype = dtype or torch.get_default_dtype()
+        device = torch.device(device) if device is not None else torch.randn(1).device
+        if dtype != torch.float16:
+            raise RuntimeError(f"unsupported data type {dtype}")
+        if device.type != "cuda":
+            raise RuntimeError("GPUKernel is enabled. But the device is not CUDA.")
+        self.n_heads, self.d_head, self.chunk_size = n_heads, d_head, chunk_size
+        self.device = device
+        self.max_chunks = max_chunks_for(memory_mb, chunk_size, n_heads, d_head, 2)
+        elems = chunk_size * n_heads * d_head * self.max_chunks
+        with torch.cuda.device(device):
+            self.key_storage = torch.empty(elems, dtype=dtype, device=device)
+            self.value_storage = torch.empty(elems, dtype=dtype, device=device)
+            self.ctx = KernelContext(n_heads, d_head, chunk_size, self.key_storage.data_ptr(),
+                                     self.value_storage.data_ptr(), self.max_chunks, tpp_threshold)
+        self.tree = Tree(chunk_size, self.max_chunks, share_prefix)
+        self._tables_version = 0
+
+    def _stream(self) -> int:
+        import torch
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _check_kv(self, t, rows: int, name: str):
+        import torch
+        if t.dtype != torch.float16 or t.device != self.device or tuple(t.shape) != (rows, self.n_heads, self.d_head):
+            raise RuntimeError(f"{name} must be fp16 [{rows}, {self.n_heads}, {self.d_head}] on {self.device}")
+        return t.contiguous()
+
+    def add_seq(self, tokens: Sequence[int], k, v) -> int:
+        k = self._check_kv(k, len(tokens), "k")
+        v = self._check_kv(v, len(tokens), "v")
+        idx, tok_begin, slots = self.tree.add_seq(tokens)
+        if slots:
+            self.ctx.scatter_kv(k.data_ptr(), v.data_ptr(), len(tokens), tok_begin, slots, self._stream())
+        self.ctx.invalidate()
+        return idx
+
+    def remove_seq(self, seq_idx: int) -> None:
+        self.tree.remove_seq(seq_idx)
+        self.ctx.invalidate()
+
+    def clear(self) -> None:
+        self.tree.clear()
+        self.ctx.invalidate()
+
+    def reserve(self) -> int:
+        n = self.tree.reserve()
+        if n:
+            self.ctx.invalidate()
+        return n
+
+    def refresh_kernel_context(self, force: bool = False) -> None:
+        if force or not self.ctx.valid:
+            self.ctx.refresh(self.tree.get_chunks(), self.tree.n_seqs, self._stream())
+
+    def append_token(self, tokens: Sequence[int], k, v, fused: bool = True) -> int:
+        if self.tree.n_seqs != len(tokens):
+            raise RuntimeError("num of seqs is not equal to num of tokens")
+        k = self._check_kv(k, len(tokens), "k")
+        v = self._check_kv(v, len(tokens), "v")
+        n_new = self.reserve()
+        self.refresh_kernel_context()
+        self.ctx.append_kv(k.data_ptr(), v.data_ptr(), len(tokens), self._stream())
+        self.tree.append_token(tokens)  # reserve inside is a no-op now
+        self.ctx.delta_tokens = self.ctx.delta_tokens + 1
+        return n_new
+
+    def forward(self, q, partition: int = 0):
+        import torch
+        if not q.is_contiguous():
+            raise RuntimeError("q is not contiguous")
+        if q.dtype != torch.float16 or q.device != self.device or q.dim() != 3 or \
+                q.shape[1] != self.n_heads or q.shape[2] != self.d_head:
+            raise RuntimeError(f"q must be fp16 [n_seqs, {self.n_heads}, {self.d_head}] on {self.device}")
+        out = torch.empty((q.shape[0], self.n_heads, self.d_head), dtype=q.dtype, device=q.device)
+        self.refresh_kernel_context()
+        self.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], partition, self._stream())
+        return out
+
+    def get_chunks(self) -> np.ndarray:
+        return self.tree.get_chunks()
+
+    def pool_views(self):
+        """(K, V) pool tensors viewed as [max_chunks, H, c, d]."""
+        shape = (self.max_chunks, self.n_heads, self.chunk_size, self.d_head)
+        return self.key_storage.view(shape), self.value_storage.view(shape)

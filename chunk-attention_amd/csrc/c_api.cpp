@@ -1,0 +1,708 @@
+// C-ABI of the decode path: kernel context (device tables, partial buffers, launches) and
+// the prefix-tree manager handle.  Declarations and their reference counterparts are in
+// include/chunk_attn_hip.h.
+#include "chunk_attn_hip.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <exception>
+#include <new>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+#include "prefix_tree.h"
+#include "tables.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int fail_hip(hipError_t e, const char* what) {
+    return fail(CA_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define CA_HIP(call)                                        \
+    do {                                                    \
+        hipError_t e_ = (call);                             \
+        if (e_ != hipSuccess) return fail_hip(e_, #call);   \
+    } while (0)
+
+// Translates C++ exceptions of the manager into error codes at the ABI boundary.
+template <typename F>
+int guarded(F&& f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc&) {
+        return fail(CA_ERR_RUNTIME, "out of host memory");
+    } catch (const std::invalid_argument& e) {
+        return fail(CA_ERR_INVALID, e.what());
+    } catch (const std::out_of_range& e) {
+        return fail(CA_ERR_INVALID, e.what());
+    } catch (const std::exception& e) {
+        const std::string msg = e.what();
+        return fail(msg.find("capacity reached") != std::string::npos ? CA_ERR_CAPACITY
+                                                                       : CA_ERR_RUNTIME,
+                    msg);
+    }
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int mb_class(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4); }
+
+}  // namespace
+
+// ---- kernel context ------------------------------------------------------------------------
+
+struct ca_ctx {
+    int H = 0, d = 0, C = 0;
+    void* k_pool = nullptr;
+    void* v_pool = nullptr;
+    int max_chunks = 0;
+    int tpp_threshold = 1;
+    int device = 0;
+    int n_cus = 256;
+    int seg_chunks = 0, stream_chunks = 0;
+
+    bool valid = false;
+    int delta_tokens = 0;
+    int partition = 0;  // partition the current plan was built for
+
+    std::vector<ca::ChunkRow> rows;  // rows of the last refresh (to rebuild for another partition)
+    int n_seqs = 0;
+    ca::RefTables ref;
+    ca::Plan plan;
+
+    // device tables: one blob, uploaded from one of two pinned staging buffers
+    char* dev_blob = nullptr;
+    size_t dev_blob_cap = 0;
+    char* host_blob[2] = { nullptr, nullptr };
+    size_t host_blob_cap[2] = { 0, 0 };
+    hipEvent_t host_blob_free[2] = { nullptr, nullptr };
+    int next_host = 0;
+    // offsets into dev_blob
+    size_t off_shared = 0, off_stream = 0, off_slots = 0, off_seq_len = 0, off_part_ptr = 0,
+           off_part_rows = 0, off_tail_slot = 0, off_tail_fill = 0;
+    int n_shared_mb[3] = { 0, 0, 0 };  // items per 16-row-block class (1, 2, 4), stored in that order
+
+    float* part = nullptr;
+    size_t part_cap = 0;  // bytes
+};
+
+namespace {
+
+int ensure_dev(char** p, size_t* cap, size_t need) {
+    if (need <= *cap) return CA_OK;
+    if (*p) CA_HIP(hipFree(*p));
+    *p = nullptr;
+    *cap = 0;
+    const size_t want = align_up(need + need / 4, 4096);
+    CA_HIP(hipMalloc(reinterpret_cast<void**>(p), want));
+    *cap = want;
+    return CA_OK;
+}
+
+ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
+    ca::LaunchArgs a;
+    a.q = q;
+    a.out = out;
+    a.kpool = c->k_pool;
+    a.vpool = c->v_pool;
+    a.part = c->part;
+    a.slots = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_slots);
+    a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
+    a.delta_tokens = c->delta_tokens;
+    a.H = c->H;
+    a.C = c->C;
+    a.scale_log2 = 1.4426950408889634f / std::sqrt(static_cast<float>(c->d));
+    return a;
+}
+
+int launch_rc(int rc, const char* what) {
+    if (rc == 0) return CA_OK;
+    if (rc < 0) return fail(CA_ERR_INVALID, std::string(what) + ": unsupported chunk_size");
+    return fail_hip(static_cast<hipError_t>(rc), what);
+}
+
+// Builds the plan for `partition` from c->rows and uploads it.
+int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
+    ca::PlanParams pp;
+    pp.tpp_threshold = c->tpp_threshold;
+    pp.partition = partition;
+    pp.shared_seg_chunks = c->seg_chunks;
+    pp.stream_chunks = c->stream_chunks;
+    pp.n_heads = c->H;
+    pp.n_cus = c->n_cus;
+    ca::build_plan(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, pp, &c->plan);
+    ca::Plan& p = c->plan;
+
+    // shared items grouped by how many 16-row blocks they need
+    std::stable_sort(p.shared_items.begin(), p.shared_items.end(),
+                     [](const ca::WorkItem& a, const ca::WorkItem& b) {
+                         return mb_class(a.n_rows) < mb_class(b.n_rows);
+                     });
+    c->n_shared_mb[0] = c->n_shared_mb[1] = c->n_shared_mb[2] = 0;
+    for (const auto& it : p.shared_items) {
+        const int mb = mb_class(it.n_rows);
+        c->n_shared_mb[mb == 1 ? 0 : (mb == 2 ? 1 : 2)]++;
+    }
+
+    size_t off = 0;
+    auto place = [&](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 64);
+        return at;
+    };
+    c->off_shared = place(p.shared_items.size() * sizeof(ca::WorkItem));
+    c->off_stream = place(p.stream_items.size() * sizeof(ca::WorkItem));
+    c->off_slots = place(p.slots.size() * 4);
+    c->off_seq_len = place(p.seq_len.size() * 4);
+    c->off_part_ptr = place(p.part_ptr.size() * 4);
+    c->off_part_rows = place(p.part_rows.size() * 4);
+    c->off_tail_slot = place(p.tail_slot.size() * 4);
+    c->off_tail_fill = place(p.tail_fill.size() * 4);
+    const size_t total = std::max<size_t>(off, 64);
+
+    if (int rc = ensure_dev(&c->dev_blob, &c->dev_blob_cap, total)) return rc;
+    const int hb = c->next_host;
+    c->next_host ^= 1;
+    // the staging buffer may still be the source of an earlier asynchronous upload
+    CA_HIP(hipEventSynchronize(c->host_blob_free[hb]));
+    if (total > c->host_blob_cap[hb]) {
+        if (c->host_blob[hb]) CA_HIP(hipHostFree(c->host_blob[hb]));
+        c->host_blob[hb] = nullptr;
+        c->host_blob_cap[hb] = 0;
+        const size_t want = align_up(total + total / 4, 4096);
+        CA_HIP(hipHostMalloc(reinterpret_cast<void**>(&c->host_blob[hb]), want, hipHostMallocDefault));
+        c->host_blob_cap[hb] = want;
+    }
+    char* hbuf = c->host_blob[hb];
+    auto put = [&](size_t at, const void* src, size_t bytes) {
+        if (bytes) std::memcpy(hbuf + at, src, bytes);
+    };
+    put(c->off_shared, p.shared_items.data(), p.shared_items.size() * sizeof(ca::WorkItem));
+    put(c->off_stream, p.stream_items.data(), p.stream_items.size() * sizeof(ca::WorkItem));
+    put(c->off_slots, p.slots.data(), p.slots.size() * 4);
+    put(c->off_seq_len, p.seq_len.data(), p.seq_len.size() * 4);
+    put(c->off_part_ptr, p.part_ptr.data(), p.part_ptr.size() * 4);
+    put(c->off_part_rows, p.part_rows.data(), p.part_rows.size() * 4);
+    put(c->off_tail_slot, p.tail_slot.data(), p.tail_slot.size() * 4);
+    put(c->off_tail_fill, p.tail_fill.data(), p.tail_fill.size() * 4);
+    CA_HIP(hipMemcpyAsync(c->dev_blob, hbuf, total, hipMemcpyHostToDevice, st));
+    CA_HIP(hipEventRecord(c->host_blob_free[hb], st));
+
+    const size_t part_bytes = std::max<size_t>(size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4, 256);
+    if (int rc = ensure_dev(reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
+    c->partition = partition;
+    return CA_OK;
+}
+
+int check_ready(ca_ctx* c, const void* q, int n_seqs) {
+    if (!c) return fail(CA_ERR_INVALID, "null context");
+    if (!c->valid) return fail(CA_ERR_STATE, "kernel context is not valid: call ca_refresh_kernel_context first");
+    if (n_seqs != c->n_seqs) {
+        return fail(CA_ERR_STATE, "n_seqs (" + std::to_string(n_seqs) + ") does not match the tables (" +
+                                    std::to_string(c->n_seqs) + ")");
+    }
+    if (n_seqs > 0 && !q) return fail(CA_ERR_INVALID, "null device pointer");
+    return CA_OK;
+}
+
+int run_shared(ca_ctx* c, const void* q, hipStream_t st) {
+    const ca::LaunchArgs a = launch_args(c, q, nullptr);
+    const ca::WorkItem* items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_shared);
+    const int mbs[3] = { 1, 2, 4 };
+    for (int k = 0; k < 3; k++) {
+        if (int rc = launch_rc(ca::launch_shared(a, items, c->n_shared_mb[k], mbs[k], st), "chunk-first launch")) return rc;
+        items += c->n_shared_mb[k];
+    }
+    return CA_OK;
+}
+
+int run_stream_and_merge(ca_ctx* c, const void* q, void* out, hipStream_t st) {
+    const ca::LaunchArgs a = launch_args(c, q, out);
+    const ca::WorkItem* items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream);
+    if (int rc = launch_rc(ca::launch_stream(a, items, static_cast<int>(c->plan.stream_items.size()), st), "sequence-first launch")) return rc;
+    if (!c->plan.part_rows.empty()) {
+        if (int rc = launch_rc(ca::launch_merge(a, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr),
+                                                reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows),
+                                                c->n_seqs, st), "merge launch")) return rc;
+    }
+    return CA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ca_last_error(void) { return g_last_error.c_str(); }
+
+int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k_pool,
+                  void* v_pool, int max_chunks, int tpp_threshold) {
+    if (!out) return fail(CA_ERR_INVALID, "null output pointer");
+    *out = nullptr;
+    if (d_head != 128) return fail(CA_ERR_INVALID, "unsupported head dim " + std::to_string(d_head));
+    if (chunk_size != 32 && chunk_size != 64 && chunk_size != 128) {
+        return fail(CA_ERR_INVALID, "unsupported chunk_size " + std::to_string(chunk_size));
+    }
+    if (n_heads <= 0 || max_chunks < 0 || tpp_threshold < 0) return fail(CA_ERR_INVALID, "bad shape argument");
+    if (max_chunks > 0 && (!k_pool || !v_pool)) return fail(CA_ERR_INVALID, "null KV pool");
+    int n_dev = 0;
+    hipError_t e = hipGetDeviceCount(&n_dev);
+    if (e != hipSuccess || n_dev <= 0) {
+        return fail(CA_ERR_HIP, "no HIP device available: the decode path has no CPU fallback");
+    }
+    return guarded([&]() -> int {
+        ca_ctx* c = new ca_ctx();
+        c->H = n_heads;
+        c->d = d_head;
+        c->C = chunk_size;
+        c->k_pool = k_pool;
+        c->v_pool = v_pool;
+        c->max_chunks = max_chunks;
+        c->tpp_threshold = tpp_threshold;
+        hipError_t err = hipGetDevice(&c->device);
+        hipDeviceProp_t prop;
+        if (err == hipSuccess) err = hipGetDeviceProperties(&prop, c->device);
+        if (err == hipSuccess) c->n_cus = prop.multiProcessorCount;
+        for (int i = 0; i < 2 && err == hipSuccess; i++) {
+            err = hipEventCreateWithFlags(&c->host_blob_free[i], hipEventDisableTiming);
+        }
+        if (err != hipSuccess) {
+            ca_ctx_destroy(c);
+            return fail_hip(err, "context setup");
+        }
+        *out = c;
+        return CA_OK;
+    });
+}
+
+void ca_ctx_destroy(ca_ctx* c) {
+    if (!c) return;
+    if (c->dev_blob) (void)hipFree(c->dev_blob);
+    if (c->part) (void)hipFree(c->part);
+    for (int i = 0; i < 2; i++) {
+        if (c->host_blob_free[i]) {
+            (void)hipEventSynchronize(c->host_blob_free[i]);
+            (void)hipEventDestroy(c->host_blob_free[i]);
+        }
+        if (c->host_blob[i]) (void)hipHostFree(c->host_blob[i]);
+    }
+    delete c;
+}
+
+int ca_refresh_kernel_context(ca_ctx* c, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                              void* stream) {
+    if (!c || n_rows < 0 || n_seqs < 0 || (n_rows > 0 && !rows)) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        static_assert(sizeof(ca_chunk_row) == sizeof(ca::ChunkRow), "row layouts must agree");
+        for (int i = 0; i < n_rows; i++) {
+            if (rows[i].slot < 0 || rows[i].slot >= c->max_chunks || rows[i].n_tokens < 0 ||
+                rows[i].n_tokens > c->C) {
+                return fail(CA_ERR_INVALID, "chunk row " + std::to_string(i) + " is outside the pool or over-full");
+            }
+        }
+        c->valid = false;
+        c->rows.resize(n_rows);
+        if (n_rows) std::memcpy(c->rows.data(), rows, sizeof(ca_chunk_row) * n_rows);
+        c->n_seqs = n_seqs;
+        ca::build_ref_tables(c->rows.data(), n_rows, n_seqs, c->C, c->tpp_threshold, &c->ref);
+        if (int rc = build_and_upload(c, 0, static_cast<hipStream_t>(stream))) return rc;
+        c->delta_tokens = 0;
+        c->valid = true;
+        return CA_OK;
+    });
+}
+
+int ca_ctx_valid(const ca_ctx* c) { return c && c->valid; }
+void ca_ctx_invalidate(ca_ctx* c) {
+    if (c) c->valid = false;
+}
+int ca_ctx_delta_tokens(const ca_ctx* c) { return c ? c->delta_tokens : 0; }
+void ca_ctx_set_delta_tokens(ca_ctx* c, int delta_tokens) {
+    if (c) c->delta_tokens = delta_tokens;
+}
+
+int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition, void* stream) {
+    if (partition < 0 || partition > 2) return fail(CA_ERR_INVALID, "Unsupported partition type");
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
+    if (n_seqs == 0) return CA_OK;
+    return guarded([&]() -> int {
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (partition != c->partition) {
+            if (int rc = build_and_upload(c, partition, st)) return rc;
+        }
+        if (int rc = run_shared(c, q, st)) return rc;
+        return run_stream_and_merge(c, q, out, st);
+    });
+}
+
+int ca_attn_chunks_first(ca_ctx* c, const void* q, int n_seqs, void* stream) {
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    return guarded([&]() -> int { return run_shared(c, q, static_cast<hipStream_t>(stream)); });
+}
+
+int ca_attn_seqs_first(ca_ctx* c, const void* q, void* out, int n_seqs, void* stream) {
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
+    return guarded([&]() -> int { return run_stream_and_merge(c, q, out, static_cast<hipStream_t>(stream)); });
+}
+
+int ca_append_kv(ca_ctx* c, const void* k, const void* v, int n_seqs, void* stream) {
+    if (int rc = check_ready(c, k, n_seqs)) return rc;
+    if (n_seqs > 0 && !v) return fail(CA_ERR_INVALID, "null device pointer");
+    for (int s = 0; s < n_seqs; s++) {
+        if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
+            return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
+        }
+    }
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    return launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
+                                       reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
+                                       n_seqs, static_cast<hipStream_t>(stream)), "append launch");
+}
+
+int ca_scatter_kv(ca_ctx* c, const void* k, const void* v, int n_tokens, int tok_begin,
+                  const int32_t* slots, int n_slots, void* stream) {
+    if (!c || n_tokens < 0 || tok_begin < 0 || n_slots < 0) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_slots == 0 || tok_begin >= n_tokens) return CA_OK;
+    if (!k || !v || !slots) return fail(CA_ERR_INVALID, "null pointer");
+    if (int64_t(n_slots) * c->C < int64_t(n_tokens - tok_begin)) {
+        return fail(CA_ERR_INVALID, "not enough chunks for the tokens to copy");
+    }
+    for (int i = 0; i < n_slots; i++) {
+        if (slots[i] < 0 || slots[i] >= c->max_chunks) return fail(CA_ERR_INVALID, "slot outside the pool");
+    }
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    return launch_rc(ca::launch_scatter(a, k, v, n_tokens, tok_begin, slots, n_slots,
+                                        static_cast<hipStream_t>(stream)), "scatter launch");
+}
+
+int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
+    if (!c || src_slot < 0 || dst_slot < 0 || src_slot >= c->max_chunks || dst_slot >= c->max_chunks) {
+        return fail(CA_ERR_INVALID, "slot outside the pool");
+    }
+    const size_t bytes = size_t(c->H) * c->C * c->d * 2;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    CA_HIP(hipMemcpyAsync(static_cast<char*>(c->k_pool) + bytes * dst_slot, static_cast<char*>(c->k_pool) + bytes * src_slot, bytes, hipMemcpyDeviceToDevice, st));
+    CA_HIP(hipMemcpyAsync(static_cast<char*>(c->v_pool) + bytes * dst_slot, static_cast<char*>(c->v_pool) + bytes * src_slot, bytes, hipMemcpyDeviceToDevice, st));
+    return CA_OK;
+}
+
+int ca_ctx_set_plan(ca_ctx* c, int shared_seg_chunks, int stream_chunks) {
+    if (!c || shared_seg_chunks < 0 || stream_chunks < 0) return fail(CA_ERR_INVALID, "bad argument");
+    c->seg_chunks = shared_seg_chunks;
+    c->stream_chunks = stream_chunks;
+    c->valid = false;
+    return CA_OK;
+}
+
+int ca_ctx_plan_info(const ca_ctx* c, ca_plan_info* info) {
+    if (!c || !info) return fail(CA_ERR_INVALID, "bad argument");
+    info->n_seqs = c->n_seqs;
+    info->n_chunks = c->ref.n_chunks;
+    info->n_shared_chunks = c->ref.n_shared;
+    info->ref_partial_rows = c->ref.partial_rows;
+    info->max_seq_n_chunks = c->ref.max_seq_n_chunks;
+    info->n_shared_items = static_cast<int>(c->plan.shared_items.size());
+    info->n_stream_items = static_cast<int>(c->plan.stream_items.size());
+    info->n_part_rows = c->plan.n_part_rows;
+    info->shared_tokens = c->plan.shared_tokens;
+    info->stream_tokens = c->plan.stream_tokens;
+    return CA_OK;
+}
+
+int ca_ctx_ref_tables(const ca_ctx* c, int32_t* final_idx, int32_t* slots, int32_t* begins,
+                      int32_t* ends, int32_t* offsets, int32_t* seq_n_tokens,
+                      int32_t* seq_chunk_map) {
+    if (!c) return fail(CA_ERR_INVALID, "null context");
+    auto copy = [](int32_t* dst, const std::vector<int32_t>& src) {
+        if (dst && !src.empty()) std::memcpy(dst, src.data(), src.size() * 4);
+    };
+    copy(final_idx, c->ref.final_idx);
+    copy(slots, c->ref.slots);
+    copy(begins, c->ref.begins);
+    copy(ends, c->ref.ends);
+    copy(offsets, c->ref.offsets);
+    copy(seq_n_tokens, c->ref.seq_n_tokens);
+    copy(seq_chunk_map, c->ref.seq_chunk_map);
+    return CA_OK;
+}
+
+int ca_ctx_export_partials(ca_ctx* c, float* maxs, float* sums, float* attns, void* stream) {
+    if (!c || !c->valid) return fail(CA_ERR_STATE, "kernel context is not valid");
+    if (c->partition != 0) return fail(CA_ERR_STATE, "partials are exported for partition 0 only");
+    return guarded([&]() -> int {
+        const ca::Plan& p = c->plan;
+        // one item group per shared chunk, in shared-chunk order, is what the layout needs
+        int n_units = 0;
+        for (const auto& it : p.shared_items) {
+            if (it.n_chunks != 1) return fail(CA_ERR_STATE, "export needs tables built with shared_seg_chunks = 1");
+            n_units++;
+        }
+        (void)n_units;
+        const size_t bytes = size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4;
+        std::vector<float> host(bytes / 4);
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (bytes) CA_HIP(hipMemcpyAsync(host.data(), c->part, bytes, hipMemcpyDeviceToHost, st));
+        CA_HIP(hipStreamSynchronize(st));
+        const float ln2 = 0.6931471805599453f;
+        // With one chunk per segment, segment k is the k-th shared chunk and its partial rows
+        // start at the reference's offsets[k]: both count n per shared chunk in row order.
+        for (int k = 0; k < c->ref.n_shared; k++) {
+            const int off = c->ref.offsets[k];
+            const int n = c->ref.ends[k] - c->ref.begins[k];
+            for (int h = 0; h < c->H; h++) {
+                for (int r = 0; r < n; r++) {
+                    const float* src = host.data() + (size_t(off + r) * c->H + h) * ca::PART_STRIDE;
+                    const size_t dst = size_t(off) * c->H + size_t(h) * n + r;
+                    if (maxs) maxs[dst] = src[0] * ln2;
+                    if (sums) sums[dst] = src[1];
+                    if (attns) std::memcpy(attns + dst * c->d, src + 4, sizeof(float) * c->d);
+                }
+            }
+        }
+        return CA_OK;
+    });
+}
+
+// ---- host-only table builder ---------------------------------------------------------------
+
+struct ca_tables {
+    ca::RefTables ref;
+    ca::Plan plan;
+    int n_seqs = 0;
+};
+
+int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                    int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks,
+                    int stream_chunks, int n_heads, int n_cus) {
+    if (!out || n_rows < 0 || n_seqs < 0 || (n_rows > 0 && !rows) || chunk_size <= 0) {
+        return fail(CA_ERR_INVALID, "bad argument");
+    }
+    if (partition < 0 || partition > 2) return fail(CA_ERR_INVALID, "Unsupported partition type");
+    return guarded([&]() -> int {
+        auto t = new ca_tables();
+        t->n_seqs = n_seqs;
+        const ca::ChunkRow* r = reinterpret_cast<const ca::ChunkRow*>(rows);
+        ca::PlanParams pp;
+        pp.tpp_threshold = tpp_threshold;
+        pp.partition = partition;
+        pp.shared_seg_chunks = shared_seg_chunks;
+        pp.stream_chunks = stream_chunks;
+        pp.n_heads = n_heads;
+        pp.n_cus = n_cus;
+        try {
+            ca::build_ref_tables(r, n_rows, n_seqs, chunk_size, tpp_threshold, &t->ref);
+            ca::build_plan(r, n_rows, n_seqs, chunk_size, pp, &t->plan);
+        } catch (...) {
+            delete t;
+            throw;
+        }
+        *out = t;
+        return CA_OK;
+    });
+}
+
+void ca_tables_destroy(ca_tables* t) { delete t; }
+
+int ca_tables_info(const ca_tables* t, ca_plan_info* info) {
+    if (!t || !info) return fail(CA_ERR_INVALID, "bad argument");
+    info->n_seqs = t->n_seqs;
+    info->n_chunks = t->ref.n_chunks;
+    info->n_shared_chunks = t->ref.n_shared;
+    info->ref_partial_rows = t->ref.partial_rows;
+    info->max_seq_n_chunks = t->ref.max_seq_n_chunks;
+    info->n_shared_items = static_cast<int>(t->plan.shared_items.size());
+    info->n_stream_items = static_cast<int>(t->plan.stream_items.size());
+    info->n_part_rows = t->plan.n_part_rows;
+    info->shared_tokens = t->plan.shared_tokens;
+    info->stream_tokens = t->plan.stream_tokens;
+    return CA_OK;
+}
+
+int ca_tables_plan_sizes(const ca_tables* t, int* n_slots, int* n_part_list) {
+    if (!t) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_slots) *n_slots = static_cast<int>(t->plan.slots.size());
+    if (n_part_list) *n_part_list = static_cast<int>(t->plan.part_rows.size());
+    return CA_OK;
+}
+
+static void copy_i32(int32_t* dst, const std::vector<int32_t>& src) {
+    if (dst && !src.empty()) std::memcpy(dst, src.data(), src.size() * 4);
+}
+
+int ca_tables_ref(const ca_tables* t, int32_t* final_idx, int32_t* slots, int32_t* begins,
+                  int32_t* ends, int32_t* offsets, int32_t* seq_n_tokens, int32_t* seq_chunk_map) {
+    if (!t) return fail(CA_ERR_INVALID, "bad argument");
+    copy_i32(final_idx, t->ref.final_idx);
+    copy_i32(slots, t->ref.slots);
+    copy_i32(begins, t->ref.begins);
+    copy_i32(ends, t->ref.ends);
+    copy_i32(offsets, t->ref.offsets);
+    copy_i32(seq_n_tokens, t->ref.seq_n_tokens);
+    copy_i32(seq_chunk_map, t->ref.seq_chunk_map);
+    return CA_OK;
+}
+
+int ca_tables_plan(const ca_tables* t, ca_work_item* shared_items, ca_work_item* stream_items,
+                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* part_rows,
+                   int32_t* tail_slot, int32_t* tail_fill) {
+    if (!t) return fail(CA_ERR_INVALID, "bad argument");
+    static_assert(sizeof(ca_work_item) == sizeof(ca::WorkItem), "work item layouts must agree");
+    if (shared_items && !t->plan.shared_items.empty()) {
+        std::memcpy(shared_items, t->plan.shared_items.data(), t->plan.shared_items.size() * sizeof(ca::WorkItem));
+    }
+    if (stream_items && !t->plan.stream_items.empty()) {
+        std::memcpy(stream_items, t->plan.stream_items.data(), t->plan.stream_items.size() * sizeof(ca::WorkItem));
+    }
+    copy_i32(slots, t->plan.slots);
+    copy_i32(seq_len, t->plan.seq_len);
+    copy_i32(part_ptr, t->plan.part_ptr);
+    copy_i32(part_rows, t->plan.part_rows);
+    copy_i32(tail_slot, t->plan.tail_slot);
+    copy_i32(tail_fill, t->plan.tail_fill);
+    return CA_OK;
+}
+
+// ---- prefix-tree manager -------------------------------------------------------------------
+
+struct ca_tree {
+    GPT::PrefixTree tree;
+    ca_tree(int c, int max_chunks, bool share) : tree(c, max_chunks, share, 0) {}
+};
+
+int ca_tree_create(ca_tree** out, int chunk_size, int max_chunks, int share_prefix) {
+    if (!out || chunk_size <= 0 || max_chunks < 0) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        *out = new ca_tree(chunk_size, max_chunks, share_prefix != 0);
+        return CA_OK;
+    });
+}
+
+void ca_tree_destroy(ca_tree* t) { delete t; }
+
+int ca_tree_max_chunks_for(int memory_mb, int chunk_size, int n_heads, int d_head, int elem_bytes) {
+    return GPT::ChunkAllocator::max_chunks_for(memory_mb, chunk_size, n_heads, d_head, elem_bytes);
+}
+
+int ca_tree_add_seq(ca_tree* t, const int32_t* tokens, int n_tokens, int* seq_idx, int* tok_begin,
+                    int32_t* new_slots, int cap, int* n_new) {
+    if (!t || n_tokens < 0 || (n_tokens > 0 && !tokens)) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        std::vector<int> ids(tokens, tokens + n_tokens);
+        std::vector<GPT::CopyJob> jobs;
+        const int idx = t->tree.add_seq(ids, &jobs);
+        if (seq_idx) *seq_idx = idx;
+        if (tok_begin) *tok_begin = jobs.empty() ? n_tokens : jobs.front().tok_begin;
+        if (n_new) *n_new = static_cast<int>(jobs.size());
+        for (int i = 0; i < static_cast<int>(jobs.size()) && i < cap && new_slots; i++) new_slots[i] = jobs[i].slot;
+        return CA_OK;
+    });
+}
+
+int ca_tree_remove_seq(ca_tree* t, int seq_idx) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        t->tree.remove_seq(seq_idx);
+        return CA_OK;
+    });
+}
+
+int ca_tree_clear(ca_tree* t) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        t->tree.clear();
+        return CA_OK;
+    });
+}
+
+int ca_tree_reserve(ca_tree* t, int* n_new) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        const auto fresh = t->tree.reserve();
+        if (n_new) *n_new = static_cast<int>(fresh.size());
+        return CA_OK;
+    });
+}
+
+int ca_tree_append_token(ca_tree* t, const int32_t* tokens, int n_tokens, int* n_new) {
+    if (!t || n_tokens < 0 || (n_tokens > 0 && !tokens)) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        if (static_cast<int>(t->tree.tails().size()) != n_tokens) {
+            throw std::runtime_error("num of seqs is not equal to num of tokens");
+        }
+        const auto fresh = t->tree.reserve();
+        t->tree.append_token_ids(std::vector<int>(tokens, tokens + n_tokens));
+        if (n_new) *n_new = static_cast<int>(fresh.size());
+        return CA_OK;
+    });
+}
+
+int ca_tree_get_chunks(const ca_tree* t, ca_chunk_row* rows, int cap, int* n_rows) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        const auto infos = t->tree.get_chunks();
+        if (n_rows) *n_rows = static_cast<int>(infos.size());
+        for (int i = 0; i < static_cast<int>(infos.size()) && i < cap && rows; i++) {
+            rows[i] = { infos[i].chunk->slot(), infos[i].chunk->n_tokens(), infos[i].seq_idx_begin, infos[i].seq_idx_end };
+        }
+        return CA_OK;
+    });
+}
+
+int ca_tree_n_seqs(const ca_tree* t) { return t ? t->tree.n_seqs() : 0; }
+int ca_tree_used_chunks(const ca_tree* t) { return t ? t->tree.allocator().used_chunks() : 0; }
+uint64_t ca_tree_version(const ca_tree* t) { return t ? t->tree.version() : 0; }
+
+int ca_tree_tails(const ca_tree* t, int32_t* slots, int cap, int* n) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    const auto& tails = t->tree.tails();
+    if (n) *n = static_cast<int>(tails.size());
+    for (int i = 0; i < static_cast<int>(tails.size()) && i < cap && slots; i++) slots[i] = tails[i]->slot();
+    return CA_OK;
+}
+
+int ca_tree_dump(const ca_tree* t, int32_t* nodes, int node_cap, int* n_nodes, int32_t* tokens,
+                 int token_cap, int* n_tokens) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        int nn = 0, nt = 0;
+        std::vector<std::pair<int, const GPT::Chunk*>> stack;
+        stack.emplace_back(0, const_cast<ca_tree*>(t)->tree.root());
+        while (!stack.empty()) {
+            const auto [depth, node] = stack.back();
+            stack.pop_back();
+            if (nodes && nn < node_cap) {
+                nodes[4 * nn + 0] = depth;
+                nodes[4 * nn + 1] = node->n_seqs;
+                nodes[4 * nn + 2] = node->n_tokens();
+                nodes[4 * nn + 3] = node->slot();
+            }
+            nn++;
+            for (int tok : node->tokens) {
+                if (tokens && nt < token_cap) tokens[nt] = tok;
+                nt++;
+            }
+            for (auto it = node->children.rbegin(); it != node->children.rend(); ++it) {
+                stack.emplace_back(depth + 1, *it);
+            }
+        }
+        if (n_nodes) *n_nodes = nn;
+        if (n_tokens) *n_tokens = nt;
+        return CA_OK;
+    });
+}
+
+}  // extern "C"

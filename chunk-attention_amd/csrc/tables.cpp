@@ -1,0 +1,219 @@
+#include "tables.h"
+
+#include <algorithm>
+#include <stdexcept>
+
+namespace ca {
+
+void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
+                      int tpp_threshold, RefTables* out) {
+    RefTables& t = *out;
+    t = RefTables();
+    t.n_chunks = n_rows;
+    // shared = covers more than tpp_threshold sequences (reference kernel_cuda.cu:1343-1349)
+    for (int i = 0; i < n_rows; i++) {
+        const int n = rows[i].seq_end - rows[i].seq_begin;
+        if (n > tpp_threshold) {
+            t.begins.push_back(rows[i].seq_begin);
+            t.ends.push_back(rows[i].seq_end);
+            t.offsets.push_back(t.partial_rows);  // exclusive prefix sum (:1358-1369)
+            t.partial_rows += n;
+        }
+    }
+    t.n_shared = static_cast<int>(t.begins.size());
+
+    t.seq_n_tokens.assign(n_seqs, 0);  // :1371-1377
+    for (int i = 0; i < n_rows; i++)
+        for (int s = rows[i].seq_begin; s < rows[i].seq_end; s++)
+            t.seq_n_tokens[s] += rows[i].n_tokens;
+    int max_len = 0;
+    for (int s = 0; s < n_seqs; s++) max_len = std::max(max_len, t.seq_n_tokens[s]);
+    t.max_seq_n_chunks = max_len / chunk_size + 1;  // :1382
+
+    // shared chunks are numbered first, both groups in row order (:1393-1410)
+    t.final_idx.resize(n_rows);
+    t.slots.assign(n_rows, -1);
+    t.seq_chunk_map.assign(size_t(n_seqs) * t.max_seq_n_chunks, -1);
+    std::vector<int> filled(n_seqs, 0);
+    int next_shared = 0, next_private = t.n_shared;
+    for (int i = 0; i < n_rows; i++) {
+        const int n = rows[i].seq_end - rows[i].seq_begin;
+        const int id = (n > tpp_threshold) ? next_shared++ : next_private++;
+        t.final_idx[i] = id;
+        t.slots[id] = rows[i].slot;
+        for (int s = rows[i].seq_begin; s < rows[i].seq_end; s++) {
+            if (filled[s] >= t.max_seq_n_chunks) {
+                throw std::logic_error("tables: a sequence has more chunks than its length allows");
+            }
+            t.seq_chunk_map[size_t(s) * t.max_seq_n_chunks + filled[s]++] = id;
+        }
+    }
+}
+
+namespace {
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+}  // namespace
+
+void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
+                const PlanParams& params, Plan* out) {
+    Plan& p = *out;
+    p = Plan();
+    p.n_seqs = n_seqs;
+    p.seq_len.assign(n_seqs, 0);
+    p.tail_slot.assign(n_seqs, -1);
+    p.tail_fill.assign(n_seqs, 0);
+
+    auto is_shared = [&](const ChunkRow& r) {
+        if (params.partition == 2) return false;
+        if (params.partition == 1) return true;
+        return (r.seq_end - r.seq_begin) > params.tpp_threshold;
+    };
+
+    // position of every row on its root->leaf path = number of chunks above it.  Rows come
+    // in pre-order, so a row's parent is the nearest earlier row whose range contains it;
+    // since every non-leaf chunk is full, position p also means "p*chunk_size tokens above".
+    std::vector<int> pos(n_rows, 0);
+    {
+        std::vector<int> depth_of_seq(n_seqs, 0);  // chunks seen so far on each sequence's path
+        for (int i = 0; i < n_rows; i++) {
+            const ChunkRow& r = rows[i];
+            if (r.seq_begin < 0 || r.seq_end > n_seqs || r.seq_begin >= r.seq_end) {
+                throw std::invalid_argument("tables: chunk row with a bad sequence range");
+            }
+            pos[i] = depth_of_seq[r.seq_begin];
+            for (int s = r.seq_begin; s < r.seq_end; s++) {
+                depth_of_seq[s]++;
+                p.seq_len[s] += r.n_tokens;
+                p.tail_slot[s] = r.slot;  // the last row covering s is its tail
+                p.tail_fill[s] = r.n_tokens;
+            }
+        }
+    }
+
+    // ---- shared runs -> segments ---------------------------------------------------------
+    struct Run { int first_row, count; };
+    std::vector<Run> runs;
+    int64_t shared_units = 0;  // (chunk, M tile) pairs
+    for (int i = 0; i < n_rows;) {
+        if (!is_shared(rows[i])) { i++; continue; }
+        int j = i + 1;
+        while (j < n_rows && is_shared(rows[j]) && rows[j].seq_begin == rows[i].seq_begin &&
+               rows[j].seq_end == rows[i].seq_end && pos[j] == pos[j - 1] + 1) {
+            j++;
+        }
+        runs.push_back({ i, j - i });
+        shared_units += int64_t(j - i) * ceil_div(rows[i].seq_end - rows[i].seq_begin, kMaxRows);
+        i = j;
+    }
+    int seg_chunks = params.shared_seg_chunks;
+    if (seg_chunks <= 0) {
+        // aim at about two workgroups per compute unit, but keep segments between 1 and 16
+        // chunks: longer segments mean fewer partial rows to write and merge
+        const int64_t target = int64_t(2) * params.n_cus;
+        const int64_t wgs_at_1 = shared_units * std::max(params.n_heads, 1);
+        seg_chunks = static_cast<int>(std::clamp<int64_t>(wgs_at_1 / std::max<int64_t>(target, 1), 1, 16));
+    }
+
+    std::vector<std::vector<int32_t>> parts_of_seq(n_seqs);
+    for (const Run& run : runs) {
+        const ChunkRow& r0 = rows[run.first_row];
+        const int n = r0.seq_end - r0.seq_begin;
+        const int n_segs = ceil_div(run.count, seg_chunks);
+        for (int g = 0; g < n_segs; g++) {
+            // spread chunks evenly over the segments of a run
+            const int c0 = int(int64_t(run.count) * g / n_segs);
+            const int c1 = int(int64_t(run.count) * (g + 1) / n_segs);
+            const int slot_first = static_cast<int>(p.slots.size());
+            for (int k = c0; k < c1; k++) {
+                p.slots.push_back(rows[run.first_row + k].slot);
+                p.shared_tokens += rows[run.first_row + k].n_tokens;
+            }
+            const int part_base = p.n_part_rows;
+            p.n_part_rows += n;
+            for (int s = 0; s < n; s++) parts_of_seq[r0.seq_begin + s].push_back(part_base + s);
+            for (int m0 = 0; m0 < n; m0 += kMaxRows) {
+                WorkItem it{};
+                it.seq_begin = r0.seq_begin + m0;
+                it.n_rows = std::min(kMaxRows, n - m0);
+                it.slot_first = slot_first;
+                it.n_chunks = c1 - c0;
+                it.part_row = part_base + m0;
+                it.pos0 = pos[run.first_row + c0];
+                it.len_seq = r0.seq_begin;
+                p.shared_items.push_back(it);
+            }
+        }
+    }
+
+    // ---- per-sequence stream items -------------------------------------------------------
+    std::vector<std::vector<int>> own_rows(n_seqs);
+    int64_t stream_chunk_total = 0;
+    for (int i = 0; i < n_rows; i++) {
+        if (is_shared(rows[i])) continue;
+        for (int s = rows[i].seq_begin; s < rows[i].seq_end; s++) {
+            own_rows[s].push_back(i);
+            stream_chunk_total++;
+        }
+    }
+    int stream_chunks = params.stream_chunks;
+    if (stream_chunks <= 0) {
+        // four waves per workgroup each take whole chunks, so prefer multiples of four;
+        // shrink towards four when there would be too few workgroups to fill the device
+        const int per_wg_tokens = 512;
+        stream_chunks = std::max(4, per_wg_tokens / chunk_size);
+        const int64_t target = int64_t(4) * params.n_cus;
+        while (stream_chunks > 4 &&
+               (stream_chunk_total / stream_chunks) * std::max(params.n_heads, 1) < target) {
+            stream_chunks /= 2;
+        }
+    }
+    for (int s = 0; s < n_seqs; s++) {
+        const auto& own = own_rows[s];
+        if (own.empty()) continue;
+        // the chunks a sequence streams are the tail end of its path: consecutive positions
+        for (size_t k = 1; k < own.size(); k++) {
+            if (pos[own[k]] != pos[own[k - 1]] + 1) {
+                throw std::logic_error("tables: private chunks of a sequence are not consecutive");
+            }
+        }
+        const int total = static_cast<int>(own.size());
+        const int n_items = ceil_div(total, stream_chunks);
+        for (int g = 0; g < n_items; g++) {
+            const int c0 = int(int64_t(total) * g / n_items);
+            const int c1 = int(int64_t(total) * (g + 1) / n_items);
+            WorkItem it{};
+            it.seq_begin = s;
+            it.n_rows = 1;
+            it.slot_first = static_cast<int>(p.slots.size());
+            it.n_chunks = c1 - c0;
+            it.pos0 = pos[own[c0]];
+            it.len_seq = s;
+            for (int k = c0; k < c1; k++) {
+                p.slots.push_back(rows[own[k]].slot);
+                p.stream_tokens += rows[own[k]].n_tokens;
+            }
+            it.part_row = p.n_part_rows++;
+            parts_of_seq[s].push_back(it.part_row);
+            p.stream_items.push_back(it);
+        }
+    }
+
+    // a sequence whose only partial comes from a stream item needs no merge: that item
+    // writes the final output itself and its partial row is dropped from the merge list
+    for (auto& it : p.stream_items) {
+        auto& parts = parts_of_seq[it.seq_begin];
+        if (parts.size() == 1) {
+            it.part_row = -1;
+            parts.clear();
+        }
+    }
+
+    p.part_ptr.assign(n_seqs + 1, 0);
+    for (int s = 0; s < n_seqs; s++) {
+        p.part_ptr[s + 1] = p.part_ptr[s] + static_cast<int>(parts_of_seq[s].size());
+        p.max_parts_per_seq = std::max(p.max_parts_per_seq, static_cast<int>(parts_of_seq[s].size()));
+        p.part_rows.insert(p.part_rows.end(), parts_of_seq[s].begin(), parts_of_seq[s].end());
+    }
+}
+
+}  // namespace ca

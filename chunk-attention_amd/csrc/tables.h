@@ -1,0 +1,83 @@
+// Flattening of the prefix tree into device tables.
+//
+// Two forms are built from the same get_chunks() rows:
+//   * RefTables: the reference's own table set (kernel_cuda.cu:1331-1445 of the reference)
+//     with K/V pointers replaced by pool slot ids.  Kept for bit-exact structure checks.
+//   * Plan: the packed work list the HIP kernels consume -- shared "segments" (runs of
+//     consecutive shared chunks covering the same sequence range, cut into pieces), per-
+//     sequence "stream" items over the chunks only that sequence reads, and per-sequence
+//     lists of the partial rows to merge.
+#pragma once
+
+#include <cstdint>
+#include <vector>
+
+namespace ca {
+
+struct ChunkRow {
+    int32_t slot;
+    int32_t n_tokens;
+    int32_t seq_begin;
+    int32_t seq_end;
+};
+
+struct RefTables {
+    int n_chunks = 0;
+    int n_shared = 0;
+    int partial_rows = 0;       // sum of n over shared chunks
+    int max_seq_n_chunks = 0;   // width of seq_chunk_map
+    std::vector<int32_t> final_idx;      // per row: chunk id after shared-first renumbering
+    std::vector<int32_t> slots;          // per final chunk id (stands for keys_values)
+    std::vector<int32_t> begins, ends, offsets;  // per shared chunk
+    std::vector<int32_t> seq_n_tokens;   // per sequence
+    std::vector<int32_t> seq_chunk_map;  // [n_seqs, max_seq_n_chunks], -1 where unwritten
+};
+
+void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
+                      int tpp_threshold, RefTables* out);
+
+// One unit of kernel work: 8 x int32 so that a wave reads it with one 32-byte scalar load.
+struct WorkItem {
+    int32_t seq_begin;   // first sequence (row of q) this item attends for
+    int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared)
+    int32_t slot_first;  // index into Plan::slots of the item's first chunk
+    int32_t n_chunks;    // consecutive entries of Plan::slots
+    int32_t part_row;    // first partial row written; -1: write the final output directly
+    int32_t pos0;        // position of the first chunk on the sequence's root->leaf path
+    int32_t len_seq;     // sequence whose length bounds the valid tokens of these chunks
+    int32_t reserved;
+};
+static_assert(sizeof(WorkItem) == 32, "WorkItem must stay 32 bytes");
+
+struct PlanParams {
+    int tpp_threshold = 1;
+    int partition = 0;        // 0: shared chunks chunk-first, rest streamed; 1: all chunk-first;
+                              // 2: everything streamed per sequence
+    int shared_seg_chunks = 0;  // max chunks per shared segment, 0 = choose from n_cus
+    int stream_chunks = 0;      // max chunks per stream item, 0 = choose from n_cus
+    int n_heads = 32;
+    int n_cus = 256;
+};
+
+constexpr int kMaxRows = 64;  // sequences per shared work item (M tile)
+
+struct Plan {
+    int n_seqs = 0;
+    int n_part_rows = 0;
+    int max_parts_per_seq = 0;
+    int64_t shared_tokens = 0;   // physical tokens attended chunk-first (per head)
+    int64_t stream_tokens = 0;   // tokens attended by stream items (per head, at build time)
+    std::vector<WorkItem> shared_items;
+    std::vector<WorkItem> stream_items;
+    std::vector<int32_t> slots;      // chunk slot lists the items index into
+    std::vector<int32_t> seq_len;    // tokens per sequence when the plan was built
+    std::vector<int32_t> part_ptr;   // [n_seqs + 1] CSR into part_rows
+    std::vector<int32_t> part_rows;  // partial rows to merge, per sequence
+    std::vector<int32_t> tail_slot;  // per sequence: slot of its last chunk
+    std::vector<int32_t> tail_fill;  // per sequence: tokens in that chunk when built
+};
+
+void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
+                const PlanParams& params, Plan* out);
+
+}  // namespace ca

@@ -1,0 +1,211 @@
+/*
+ * C-ABI of the MI355X ChunkAttention decode path (libchunkattn_hip.so).
+ *
+ * Plain C types and raw pointers only.  Pointers named *_dev / q / out / k / v / *_pool are
+ * device (HBM) addresses; everything else is host memory.  `stream` is a hipStream_t passed
+ * as void* (NULL = the default stream).  Every function returns 0 on success or a negative
+ * CA_ERR_* code; ca_last_error() gives the message for the calling thread.
+ *
+ * Two groups of entry points:
+ *   ca_ctx_*, ca_refresh_kernel_context, ca_attention, ca_attn_chunks_first,
+ *   ca_attn_seqs_first, ca_append_kv: the kernel seam.  They replace the functions the
+ *   reference declares in cpp/chunk_attn/kernel_cuda.h:57-71 and its KernelContext
+ *   (kernel_cuda.h:9-55), with torch tensors replaced by pointers and chunk pointers by pool
+ *   slot ids.
+ *   ca_tree_*: the prefix-tree chunk manager (reference cpp/chunk_attn/attention.cpp), for
+ *   hosts that do not link the C++ class.
+ *
+ * Layouts (fp16, d_head = 128):
+ *   q, out          [n_seqs, n_heads, d_head]
+ *   k, v (add)      [n_tokens, n_heads, d_head]
+ *   k, v (append)   [n_seqs, n_heads, d_head]
+ *   k_pool, v_pool  [max_chunks][n_heads][chunk_size][d_head]; chunk `slot` starts at element
+ *                   slot * n_heads * chunk_size * d_head
+ */
+#ifndef CHUNK_ATTN_HIP_H
+#define CHUNK_ATTN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CA_OK 0
+#define CA_ERR_INVALID (-1)   /* bad argument / unsupported shape */
+#define CA_ERR_HIP (-2)       /* a HIP runtime call failed */
+#define CA_ERR_STATE (-3)     /* tables not valid, sizes do not match the tables, ... */
+#define CA_ERR_CAPACITY (-4)  /* chunk pool exhausted */
+#define CA_ERR_RUNTIME (-5)   /* other manager errors (message says which) */
+
+const char* ca_last_error(void);
+
+/* ---- kernel context ------------------------------------------------------------------- */
+
+typedef struct ca_ctx ca_ctx;
+
+/* One flattened-tree row: reference ChunkInfo (cpp/chunk_attn/chunk_info.h:6-15) with the
+ * Chunk* replaced by the chunk's pool slot and token count. */
+typedef struct ca_chunk_row {
+    int32_t slot;
+    int32_t n_tokens;
+    int32_t seq_begin;
+    int32_t seq_end;
+} ca_chunk_row;
+
+/* Replaces KernelContext's constructor (kernel_cuda.h:10-31).  d_head must be 128 and
+ * chunk_size one of 32, 64, 128, as in the reference (kernel_cuda.cu:1199, 1256-1265).
+ * The pools stay owned by the caller and must outlive the context. */
+int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k_pool,
+                  void* v_pool, int max_chunks, int tpp_threshold);
+void ca_ctx_destroy(ca_ctx* ctx);
+
+/* Replaces refresh_kernel_context(ctx, chunk_infos, n_seqs) (kernel_cuda.cu:1331-1445):
+ * flattens the rows (in get_chunks order) into device tables, sizes the partial-result
+ * buffer, resets delta_tokens to 0 and marks the context valid. */
+int ca_refresh_kernel_context(ca_ctx* ctx, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                              void* stream);
+
+/* KernelContext::valid / delta_tokens (kernel_cuda.h:42-45). */
+int ca_ctx_valid(const ca_ctx* ctx);
+void ca_ctx_invalidate(ca_ctx* ctx);
+int ca_ctx_delta_tokens(const ca_ctx* ctx);
+void ca_ctx_set_delta_tokens(ca_ctx* ctx, int delta_tokens);
+
+/* Replaces attention(ctx, q, out, partition) (kernel_cuda.cu:1320-1329).  partition 0:
+ * chunks covering more than tpp_threshold sequences are attended chunk-first, the rest per
+ * sequence; 1: every chunk chunk-first; 2: every chunk per sequence (the meaning the
+ * reference's CPU path gives the argument, kernel_cpu_mkl.cpp:364-372). */
+int ca_attention(ca_ctx* ctx, const void* q, void* out, int n_seqs, int partition,
+                 void* stream);
+
+/* Replaces attn_chunks_first(ctx, q) (kernel_cuda.cu:1118-1193): partial (max, sum, P.V)
+ * of every shared segment into the context's partial buffer. */
+int ca_attn_chunks_first(ca_ctx* ctx, const void* q, int n_seqs, void* stream);
+
+/* Replaces attn_seqs_first(ctx, q, out) (kernel_cuda.cu:1195-1271): streams every
+ * sequence's own chunks, merges them with the partials of ca_attn_chunks_first and writes
+ * the normalised output. */
+int ca_attn_seqs_first(ca_ctx* ctx, const void* q, void* out, int n_seqs, void* stream);
+
+/* Replaces append_kv(ctx, keys, values) (kernel_cuda.cu:1273-1318): writes one new K/V row
+ * per sequence at position seq_len + delta_tokens.  Does not change delta_tokens. */
+int ca_append_kv(ca_ctx* ctx, const void* k, const void* v, int n_seqs, void* stream);
+
+/* Copy-in of an inserted sequence's K/V (what the reference does with two tensor slice
+ * assignments per chunk, cpp/chunk_attn/chunk.cpp:63-72): token rows
+ * [tok_begin, tok_begin + n_slots*chunk_size) clipped to n_tokens go to the listed chunks,
+ * chunk_size rows each, starting at row 0.  k, v: [n_tokens, n_heads, d_head]. */
+int ca_scatter_kv(ca_ctx* ctx, const void* k, const void* v, int n_tokens, int tok_begin,
+                  const int32_t* slots, int n_slots, void* stream);
+
+/* Device copy of one chunk's K and V (reference Chunk::deep_copy, chunk.cpp:93-107). */
+int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
+
+/* Work-list shaping.  0 = choose from the device's compute-unit count.
+ * shared_seg_chunks = 1 gives one partial row set per shared chunk, the granularity of the
+ * reference's partial buffers. */
+int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
+
+/* Numbers describing the current tables. */
+typedef struct ca_plan_info {
+    int32_t n_seqs;
+    int32_t n_chunks;           /* rows given to the last refresh */
+    int32_t n_shared_chunks;    /* reference n_shared_chunks */
+    int32_t ref_partial_rows;   /* reference partial_attn_dim (sum of n over shared chunks) */
+    int32_t max_seq_n_chunks;   /* width of the reference seq_chunk_map */
+    int32_t n_shared_items;
+    int32_t n_stream_items;
+    int32_t n_part_rows;
+    int64_t shared_tokens;      /* physical tokens attended chunk-first */
+    int64_t stream_tokens;      /* tokens streamed per sequence (when the tables were built) */
+} ca_plan_info;
+int ca_ctx_plan_info(const ca_ctx* ctx, ca_plan_info* info);
+
+/* Reference-form tables of the last refresh, copied into caller buffers (NULL = skip):
+ *   final_idx [n_chunks], slots [n_chunks], begins/ends/offsets [n_shared_chunks],
+ *   seq_n_tokens [n_seqs], seq_chunk_map [n_seqs * max_seq_n_chunks] (-1 = unwritten). */
+int ca_ctx_ref_tables(const ca_ctx* ctx, int32_t* final_idx, int32_t* slots, int32_t* begins,
+                      int32_t* ends, int32_t* offsets, int32_t* seq_n_tokens,
+                      int32_t* seq_chunk_map);
+
+/* Copies the chunk-first partials to host buffers in the reference's layout
+ * (kernel_cuda.cu:830-838): for shared chunk i with n covered sequences and row offset
+ * off = offsets[i]:  maxs/sums[off*H + h*n + r], attns[(off*H + h*n + r)*d ...], maxima in
+ * natural-log units of score/sqrt(d).  Needs tables built with shared_seg_chunks = 1 and
+ * partition 0.  Synchronises the stream. */
+int ca_ctx_export_partials(ca_ctx* ctx, float* maxs, float* sums, float* attns, void* stream);
+
+/* ---- host-only table builder (no device needed) ---------------------------------------- */
+
+/* The flattening ca_refresh_kernel_context performs, exposed for structure checks: builds
+ * the reference-form tables (kernel_cuda.cu:1331-1445) and the packed work list from the
+ * rows, entirely on the host. */
+typedef struct ca_tables ca_tables;
+
+/* One unit of kernel work (see csrc/tables.h). */
+typedef struct ca_work_item {
+    int32_t seq_begin, n_rows, slot_first, n_chunks, part_row, pos0, len_seq, reserved;
+} ca_work_item;
+
+int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                    int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks,
+                    int stream_chunks, int n_heads, int n_cus);
+void ca_tables_destroy(ca_tables* t);
+/* sizes: fills the same struct ca_ctx_plan_info fills */
+int ca_tables_info(const ca_tables* t, ca_plan_info* info);
+/* lengths of the variable-size plan arrays: n_slots, n_part_list */
+int ca_tables_plan_sizes(const ca_tables* t, int* n_slots, int* n_part_list);
+/* reference-form tables, same buffers as ca_ctx_ref_tables */
+int ca_tables_ref(const ca_tables* t, int32_t* final_idx, int32_t* slots, int32_t* begins,
+                  int32_t* ends, int32_t* offsets, int32_t* seq_n_tokens, int32_t* seq_chunk_map);
+/* packed plan: shared_items [n_shared_items], stream_items [n_stream_items], slots [n_slots],
+ * seq_len / tail_slot / tail_fill [n_seqs], part_ptr [n_seqs + 1], part_rows [n_part_list] */
+int ca_tables_plan(const ca_tables* t, ca_work_item* shared_items, ca_work_item* stream_items,
+                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* part_rows,
+                   int32_t* tail_slot, int32_t* tail_fill);
+
+/* ---- prefix-tree chunk manager -------------------------------------------------------- */
+
+typedef struct ca_tree ca_tree;
+
+/* reference Attention's tree state + ChunkAllocator (attention.cpp:8-37,
+ * chunk_allocator.cpp:8-56), without tensors. */
+int ca_tree_create(ca_tree** out, int chunk_size, int max_chunks, int share_prefix);
+void ca_tree_destroy(ca_tree* tree);
+/* reference ChunkAllocator's capacity rule (chunk_allocator.cpp:32-35). */
+int ca_tree_max_chunks_for(int memory_mb, int chunk_size, int n_heads, int d_head,
+                           int elem_bytes);
+
+/* reference Attention::add_seq (attention.cpp:141-193).  *seq_idx: index the sequence was
+ * inserted at.  new_slots (capacity cap) receives the slots of the chunks that need K/V
+ * copied in, in order; they hold tokens [*tok_begin, n_tokens).  *n_new may exceed cap, in
+ * which case only cap entries were written. */
+int ca_tree_add_seq(ca_tree* tree, const int32_t* tokens, int n_tokens, int* seq_idx,
+                    int* tok_begin, int32_t* new_slots, int cap, int* n_new);
+/* reference Attention::remove_seq (attention.cpp:263-278) */
+int ca_tree_remove_seq(ca_tree* tree, int seq_idx);
+int ca_tree_clear(ca_tree* tree);
+/* reference Attention::reserve (attention.cpp:116-131); *n_new = chunks added */
+int ca_tree_reserve(ca_tree* tree, int* n_new);
+/* host half of reference Attention::append_token (attention.cpp:80-114): reserve, then
+ * record one token id per sequence.  Returns *n_new like ca_tree_reserve. */
+int ca_tree_append_token(ca_tree* tree, const int32_t* tokens, int n_tokens, int* n_new);
+/* reference Attention::get_chunks (attention.cpp:342-372).  Writes up to cap rows and
+ * returns the total number of rows in *n_rows. */
+int ca_tree_get_chunks(const ca_tree* tree, ca_chunk_row* rows, int cap, int* n_rows);
+int ca_tree_n_seqs(const ca_tree* tree);
+int ca_tree_used_chunks(const ca_tree* tree);
+uint64_t ca_tree_version(const ca_tree* tree);
+/* slot of the tail chunk of every sequence, in sequence order (reference tails()) */
+int ca_tree_tails(const ca_tree* tree, int32_t* slots, int cap, int* n);
+/* Pre-order dump (children first-to-last) of the whole tree for structure checks: per node
+ * 4 ints (depth, n_seqs, n_tokens, slot; the root has slot -1) and its tokens appended to
+ * `tokens`.  Returns counts in *n_nodes / *n_tokens; writes at most the given capacities. */
+int ca_tree_dump(const ca_tree* tree, int32_t* nodes, int node_cap, int* n_nodes,
+                 int32_t* tokens, int token_cap, int* n_tokens);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CHUNK_ATTN_HIP_H */

@@ -1,0 +1,142 @@
+"""Device-table flattening (host side of ca_refresh_kernel_context): reference-form tables
+bit-exact against the oracle and the hand-worked example; structural invariants of the packed
+work list the kernels consume."""
+import random
+
+import numpy as np
+import pytest
+
+from chunk_attn import capi, synth
+from oracle.prefix_tree import PrefixTree, build_ref_tables
+from kats import ADD_SEQ_STEPS, TABLE_KAT
+
+
+def rows_np(tree: PrefixTree):
+    return np.array([r.as_tuple() for r in tree.get_chunks()], np.int32).reshape(-1, 4)
+
+
+def assert_ref_equal(ref: dict, want):
+    assert ref["n_shared"] == want.n_shared
+    assert ref["partial_rows"] == want.partial_rows
+    assert ref["max_seq_n_chunks"] == want.max_seq_n_chunks
+    np.testing.assert_array_equal(ref["final_idx"], want.final_idx)
+    np.testing.assert_array_equal(ref["slots"], want.slots)
+    np.testing.assert_array_equal(ref["begins"], want.begins)
+    np.testing.assert_array_equal(ref["ends"], want.ends)
+    np.testing.assert_array_equal(ref["offsets"], want.offsets)
+    np.testing.assert_array_equal(ref["seq_n_tokens"], want.seq_n_tokens)
+    np.testing.assert_array_equal(ref["seq_chunk_map"], np.array(want.seq_chunk_map, np.int32).reshape(
+        ref["seq_chunk_map"].shape))
+
+
+def test_table_kat():
+    t = PrefixTree(2, 64)
+    for tokens, _, _ in ADD_SEQ_STEPS:
+        t.add_seq(tokens)
+    tabs = capi.build_tables(rows_np(t), t.n_seqs, 2, 1)["ref"]
+    for key in ("final_idx", "begins", "ends", "offsets", "seq_n_tokens"):
+        assert tabs[key].tolist() == TABLE_KAT[key]
+    assert tabs["seq_chunk_map"].tolist() == TABLE_KAT["seq_chunk_map"]
+    assert (tabs["n_shared"], tabs["partial_rows"], tabs["max_seq_n_chunks"]) == (2, 9, 3)
+
+
+def check_plan(rows, n_seqs, c, plan, tpp, partition):
+    """Every (sequence, chunk) pair is attended exactly once, in path order; partial lists
+    name exactly the rows the items write."""
+    covered = {s: [] for s in range(n_seqs)}        # s -> list of (pos, slot)
+    written = {}                                    # part_row -> seq
+    slots = plan["slots"]
+    for it in plan["shared_items"]:
+        b, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
+        assert 1 <= n <= 64 and nc >= 1
+        for i in range(n):
+            assert pr + i not in written
+            written[pr + i] = b + i
+            for k in range(nc):
+                covered[b + i].append((pos0 + k, int(slots[sf + k])))
+    for it in plan["stream_items"]:
+        s, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
+        assert n == 1 and lseq == s and nc >= 1
+        if pr >= 0:
+            assert pr not in written
+            written[pr] = s
+        for k in range(nc):
+            covered[s].append((pos0 + k, int(slots[sf + k])))
+    # expected coverage from the rows
+    want = {s: [] for s in range(n_seqs)}
+    depth = [0] * n_seqs
+    for (slot, nt, b, e) in rows.tolist():
+        for s in range(b, e):
+            want[s].append((depth[s], slot))
+            depth[s] += 1
+    for s in range(n_seqs):
+        assert sorted(covered[s]) == want[s]
+        lst = plan["part_rows"][plan["part_ptr"][s]:plan["part_ptr"][s + 1]].tolist()
+        mine = sorted(r for r, q in written.items() if q == s)
+        direct = [it for it in plan["stream_items"] if it[0] == s and it[4] < 0]
+        if direct:
+            assert lst == [] and mine == [] and len(direct) == 1
+        else:
+            assert sorted(lst) == mine and len(mine) >= 1
+        assert plan["seq_len"][s] == sum(nt for (_, nt, b, e) in rows.tolist() if b <= s < e)
+        last = [r for r in rows.tolist() if r[2] <= s < r[3]][-1]
+        assert (plan["tail_slot"][s], plan["tail_fill"][s]) == (last[0], last[1])
+    assert all(0 <= r < plan["n_part_rows"] for r in written)
+    if partition == 2:
+        assert len(plan["shared_items"]) == 0
+    if partition == 1:
+        assert len(plan["stream_items"]) == 0
+    if partition == 0:
+        for it in plan["shared_items"]:
+            pass
+        shared_rows = rows[(rows[:, 3] - rows[:, 2]) > tpp]
+        assert plan["shared_tokens"] == int(shared_rows[:, 1].sum())
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_trees(seed):
+    rng = random.Random(seed)
+    c = rng.choice([2, 4])
+    t = PrefixTree(c, 4096)
+    n = 0
+    for _ in range(60):
+        op = rng.random()
+        if op < 0.6 or n == 0:
+            t.add_seq([rng.randint(0, 1) for _ in range(rng.randint(1, 4 * c))])
+            n += 1
+        elif op < 0.85:
+            t.append_token([rng.randint(0, 1) for _ in range(n)])
+        else:
+            t.remove_seq(rng.randrange(n))
+            n -= 1
+    rows = rows_np(t)
+    for tpp in (0, 1, 2):
+        for partition in (0, 1, 2):
+            for seg, strm in ((0, 0), (1, 1), (3, 2)):
+                out = capi.build_tables(rows, t.n_seqs, c, tpp, partition, seg, strm, n_heads=4, n_cus=8)
+                assert_ref_equal(out["ref"], build_ref_tables(rows.tolist(), t.n_seqs, c, tpp))
+                check_plan(rows, t.n_seqs, c, out["plan"], tpp, partition)
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 3])
+def test_benchmark_plans(cfg):
+    w = synth.baseline_config(cfg)
+    need = sum(w.seq_len(s) // w.chunk_size + 2 for s in range(w.n_seqs))
+    t = PrefixTree(w.chunk_size, need)
+    for s in range(w.n_seqs):
+        t.add_seq(w.tokens(s))
+    rows = rows_np(t)
+    out = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0)
+    assert_ref_equal(out["ref"], build_ref_tables(rows.tolist(), t.n_seqs, w.chunk_size, 1))
+    check_plan(rows, t.n_seqs, w.chunk_size, out["plan"], 1, 0)
+    assert out["plan"]["shared_tokens"] == w.shared_tokens_physical()
+    assert out["plan"]["stream_tokens"] == w.logical_tokens() - w.n_seqs * sum(
+        len(seg.ids) for seg in w.seqs[0] if seg.k_stream < synth.STREAM_K_UNIQUE)
+
+
+def test_bad_rows_rejected():
+    rows = np.array([[0, 2, 0, 3]], np.int32)
+    with pytest.raises(capi.ChunkAttnError):
+        capi.build_tables(rows, 2, 2)          # range exceeds n_seqs
+    with pytest.raises(capi.ChunkAttnError):
+        capi.build_tables(rows, 3, 2, partition=5)
