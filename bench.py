@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Decode-attention benchmark on one MI355X.
+
+One "step" = one forward of the prefix-tree decode attention (chunk-first launches +
+sequence-first launch + merge) over a synthetic batch whose K/V already sit in the HBM pool
+and whose device tables are valid -- the protocol of the reference's own microbenchmark
+(tests/benchmark_chunk_attn.py:60-97 there: warm-up, then timed forwards between device syncs).
+
+Prints one JSON line: metric = decode-attention us/step (lower is better) with the achieved
+HBM rate of the dominant kernel against the 8 TB/s roofline and the CPU baseline next to it.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "chunk-attention_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def build_cache(w, torch, capi, seed=0, tpp_threshold=1):
+    import numpy as np
+    dev = torch.device("cuda:0")
+    need = sum(w.seq_len(s) // w.chunk_size + 2 for s in range(w.n_seqs)) + 8
+    per_chunk = w.chunk_size * w.n_heads * w.d_head * 2 * 2
+    memory_mb = -(-need * per_chunk // (1 << 20))
+    attn = capi.Attention(n_heads=w.n_heads, d_head=w.d_head, chunk_size=w.chunk_size, memory_mb=memory_mb,
+                          share_prefix=True, tpp_threshold=tpp_threshold, dtype=torch.float16, device=dev)
+    for s in range(w.n_seqs):
+        k, v = w.kv(s, seed)
+        idx = attn.add_seq(w.tokens(s), torch.from_numpy(np.ascontiguousarray(k)).to(dev),
+                           torch.from_numpy(np.ascontiguousarray(v)).to(dev))
+        assert idx == s
+    return attn
+
+
+def time_forward(attn, q, out, steps, warmup, torch, partition=0):
+    stream = torch.cuda.current_stream().cuda_stream
+    n = q.shape[0]
+    attn.refresh_kernel_context()
+    for _ in range(warmup):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), n, partition, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), n, partition, stream)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def phase_times(attn, q, out, steps, torch, partition=0):
+    stream = torch.cuda.current_stream().cuda_stream
+    attn.ctx.set_timing(True)
+    attn.ctx.read_timing(reset=True)
+    for _ in range(steps):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], partition, stream)
+    t = attn.ctx.read_timing(reset=True)
+    attn.ctx.set_timing(False)
+    n = max(t["calls"], 1)
+    return {k: t[k] / n for k in ("shared_ms", "stream_ms", "merge_ms")}
+
+
+def cpu_baseline(attn, q_np, budget_s, torch):
+    """The CPU restatement of the reference's MKL path on the same cache contents (fp16 values
+    widened to fp32), timed on this machine's host cores."""
+    import numpy as np
+    from oracle.attention_ref import CpuAttention
+    rows = attn.get_chunks()
+    top = int(rows[:, 0].max()) + 1
+    kp, vp = attn.pool_views()
+    kpool = kp[:top].float().cpu().numpy()
+    vpool = vp[:top].float().cpu().numpy()
+    cpu = CpuAttention("auto")
+    threads = min(cpu.max_threads, torch.get_num_threads())
+    qf = q_np.astype(np.float32)
+    res = {}
+    for name, part in (("chunk_first", 0), ("seq_first", 2)):
+        cpu.attention(qf, rows, kpool, vpool, part, threads)  # warm-up
+        n, t0 = 0, time.perf_counter()
+        while True:
+            ref = cpu.attention(qf, rows, kpool, vpool, part, threads)
+            n += 1
+            el = time.perf_counter() - t0
+            if el > budget_s / 2 or n >= 100:
+                break
+        res[name] = (el / n * 1e6, n)
+    return res, threads, cpu.blas_source, ref
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=1, help="0-based index into the benchmark configurations (default: batch 32, 2048 shared + 512 unique, chunk 64)")
+    ap.add_argument("--fraction", type=float, default=0.5, help="shared fraction for configuration 2")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget, 0 to skip")
+    ap.add_argument("--no-paged", action="store_true", help="skip the private-copies baseline")
+    ap.add_argument("--seg-chunks", type=int, default=0)
+    ap.add_argument("--stream-chunks", type=int, default=0)
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the decode path has no multi-GPU component (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    from chunk_attn import capi, synth
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X: no HIP device visible and there is no CPU fallback", file=sys.stderr)
+        return 3
+    torch.cuda.set_device(0)
+
+    w = synth.baseline_config(args.config, args.fraction)
+    attn = build_cache(w, torch, capi, args.seed)
+    if args.seg_chunks or args.stream_chunks:
+        attn.ctx.set_plan(args.seg_chunks, args.stream_chunks)
+    q_np = w.q(args.seed)
+    q = torch.from_numpy(q_np).to("cuda:0")
+    out = torch.empty_like(q)
+
+    ms = time_forward(attn, q, out, args.steps, args.warmup, torch)
+    ph = phase_times(attn, q, out, min(args.steps, 100), torch)
+    info = attn.ctx.plan_info()
+    H, d = w.n_heads, w.d_head
+    tok_bytes = 4 * H * d  # K and V rows of one token, all heads, fp16
+    stream_bytes = tok_bytes * info.stream_tokens
+    shared_bytes = tok_bytes * info.shared_tokens
+    qo_bytes = 4 * w.n_seqs * H * d
+    step_bytes = stream_bytes + shared_bytes + qo_bytes
+    if ph["stream_ms"] >= ph["shared_ms"]:
+        dom, dom_ms, dom_bytes = "stream_kernel", ph["stream_ms"], stream_bytes
+    else:
+        dom, dom_ms, dom_bytes = "shared_kernel", ph["shared_ms"], shared_bytes
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+
+    result = {
+        "metric": "decode attention us/step",
+        "value": round(ms * 1e3, 3),
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": w.name, "n_seqs": w.n_seqs, "n_heads": H, "d_head": d, "chunk_size": w.chunk_size,
+                   "shared_tokens": int(info.shared_tokens), "stream_tokens": int(info.stream_tokens),
+                   "shared_items": info.n_shared_items, "stream_items": info.n_stream_items,
+                   "partial_rows": info.n_part_rows},
+        "step_bytes": step_bytes,
+        "step_GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+        "step_frac_of_hbm_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "phases_us": {k.replace("_ms", ""): round(v * 1e3, 2) for k, v in ph.items()},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_ms * 1e3, 2)},
+    }
+
+    if not args.no_paged:
+        pw = synth.paged_variant(w)
+        pattn = build_cache(pw, torch, capi, args.seed)
+        pout = torch.empty_like(q)
+        pms = time_forward(pattn, q, pout, max(args.steps // 4, 10), max(args.warmup // 4, 2), torch)
+        logical = tok_bytes * w.logical_tokens()
+        physical = stream_bytes + shared_bytes
+        torch.cuda.synchronize()
+        diff = float((pout.float() - out.float()).abs().max())
+        result["paged_baseline"] = {"us_per_step": round(pms * 1e3, 2), "speedup": round(pms / ms, 3),
+                                    "kv_sharing_ratio": round(logical / physical, 3),
+                                    "GBps": round((logical + qo_bytes) / (pms * 1e-3) / 1e9, 1),
+                                    "max_abs_diff_vs_shared": diff}
+        del pattn
+
+    if args.cpu_seconds > 0:
+        res, threads, blas, ref = cpu_baseline(attn, q_np, args.cpu_seconds, torch)
+        err = float(np.abs(out.float().cpu().numpy() - ref).max())
+        result["cpu_baseline"] = {"value": round(res["chunk_first"][0], 1), "unit": "us/step", "cores": threads,
+                                  "kind": "port",
+                                  "sample": "%s, full workload, fp32; chunk-first x%d forwards (value), sequence-first x%d forwards = %.1f us/step; host has %d logical cpus; %s" % (
+                                      w.name, res["chunk_first"][1], res["seq_first"][1], res["seq_first"][0],
+                                      os.cpu_count(), blas)}
+        result["max_abs_err_vs_cpu"] = err
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -62,6 +62,10 @@ SIGNATURES = {
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
+    "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_ctx_read_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double),
+                                          ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
+                                          ctypes.POINTER(ctypes.c_int64), ctypes.c_int]),
     "ca_ctx_plan_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
     "ca_ctx_ref_tables": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
     "ca_ctx_export_partials": (ctypes.c_int, [ctypes.c_void_p, c_f32_p, c_f32_p, c_f32_p,
@@ -340,6 +344,17 @@ class KernelContext:
 
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
+
+    def set_timing(self, enable: bool) -> None:
+        _check(self._lib.ca_ctx_set_timing(self._h, int(enable)))
+
+    def read_timing(self, reset: bool = True) -> dict:
+        """Accumulated per-phase milliseconds of the timed ca_attention calls."""
+        a, b, c = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        n = ctypes.c_int64()
+        _check(self._lib.ca_ctx_read_timing(self._h, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c),
+                                            ctypes.byref(n), int(reset)))
+        return {"shared_ms": a.value, "stream_ms": b.value, "merge_ms": c.value, "calls": n.value}
 
     def plan_info(self) -> PlanInfo:
         info = PlanInfo()

@@ -65,6 +65,7 @@ class Workload:
     sigma: float
     seqs: List[List[Segment]] = field(default_factory=list)
     append_steps: int = 0
+    _cache: Dict[Tuple[int, int, int], np.ndarray] = field(default_factory=dict, repr=False)
 
     @property
     def n_seqs(self) -> int:
@@ -79,12 +80,16 @@ class Workload:
     def kv(self, s: int, seed: int = 0) -> Tuple[np.ndarray, np.ndarray]:
         """K, V of sequence s as fp16 [T, H, d].  Shared segments regenerate the same values
         for every sequence that contains them."""
-        hd = self.n_heads * self.d_head
-        ks, vs = [], []
-        for seg in self.seqs[s]:
-            ks.append(normal_fp16(seed, seg.k_stream, (len(seg.ids), self.n_heads, self.d_head), self.sigma))
-            vs.append(normal_fp16(seed, seg.v_stream, (len(seg.ids), self.n_heads, self.d_head), self.sigma))
-        del hd
+        def draw(stream: int, n: int) -> np.ndarray:
+            if stream >= STREAM_K_UNIQUE:
+                return normal_fp16(seed, stream, (n, self.n_heads, self.d_head), self.sigma)
+            key = (seed, stream, n)  # shared segments are drawn once
+            if key not in self._cache:
+                self._cache[key] = normal_fp16(seed, stream, (n, self.n_heads, self.d_head), self.sigma)
+            return self._cache[key]
+
+        ks = [draw(seg.k_stream, len(seg.ids)) for seg in self.seqs[s]]
+        vs = [draw(seg.v_stream, len(seg.ids)) for seg in self.seqs[s]]
         return np.concatenate(ks, axis=0), np.concatenate(vs, axis=0)
 
     def q(self, seed: int = 0) -> np.ndarray:

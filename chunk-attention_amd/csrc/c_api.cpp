@@ -97,6 +97,13 @@ struct ca_ctx {
 
     float* part = nullptr;
     size_t part_cap = 0;  // bytes
+
+    // optional per-phase timing: events recorded on the caller's stream around the launches
+    bool timing = false;
+    hipEvent_t ev[4] = { nullptr, nullptr, nullptr, nullptr };
+    bool ev_pending = false;
+    double phase_ms[3] = { 0, 0, 0 };
+    int64_t phase_calls = 0;
 };
 
 namespace {
@@ -218,6 +225,20 @@ int check_ready(ca_ctx* c, const void* q, int n_seqs) {
     return CA_OK;
 }
 
+// Adds the elapsed times of the last timed ca_attention call to the accumulators.
+int collect_timing(ca_ctx* c) {
+    if (!c->ev_pending) return CA_OK;
+    CA_HIP(hipEventSynchronize(c->ev[3]));
+    for (int i = 0; i < 3; i++) {
+        float ms = 0.f;
+        CA_HIP(hipEventElapsedTime(&ms, c->ev[i], c->ev[i + 1]));
+        c->phase_ms[i] += ms;
+    }
+    c->phase_calls++;
+    c->ev_pending = false;
+    return CA_OK;
+}
+
 int run_shared(ca_ctx* c, const void* q, hipStream_t st) {
     const ca::LaunchArgs a = launch_args(c, q, nullptr);
     const ca::WorkItem* items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_shared);
@@ -298,6 +319,9 @@ void ca_ctx_destroy(ca_ctx* c) {
         }
         if (c->host_blob[i]) (void)hipHostFree(c->host_blob[i]);
     }
+    for (int i = 0; i < 4; i++) {
+        if (c->ev[i]) (void)hipEventDestroy(c->ev[i]);
+    }
     delete c;
 }
 
@@ -343,9 +367,54 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
         if (partition != c->partition) {
             if (int rc = build_and_upload(c, partition, st)) return rc;
         }
+        if (!c->timing) {
+            if (int rc = run_shared(c, q, st)) return rc;
+            return run_stream_and_merge(c, q, out, st);
+        }
+        if (int rc = collect_timing(c)) return rc;
+        const ca::LaunchArgs a = launch_args(c, q, out);
+        CA_HIP(hipEventRecord(c->ev[0], st));
         if (int rc = run_shared(c, q, st)) return rc;
-        return run_stream_and_merge(c, q, out, st);
+        CA_HIP(hipEventRecord(c->ev[1], st));
+        if (int rc = launch_rc(ca::launch_stream(a, reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream),
+                                                 static_cast<int>(c->plan.stream_items.size()), st), "sequence-first launch")) return rc;
+        CA_HIP(hipEventRecord(c->ev[2], st));
+        if (!c->plan.part_rows.empty()) {
+            if (int rc = launch_rc(ca::launch_merge(a, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr),
+                                                    reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows),
+                                                    c->n_seqs, st), "merge launch")) return rc;
+        }
+        CA_HIP(hipEventRecord(c->ev[3], st));
+        c->ev_pending = true;
+        return CA_OK;
     });
+}
+
+int ca_ctx_set_timing(ca_ctx* c, int enable) {
+    if (!c) return fail(CA_ERR_INVALID, "null context");
+    if (enable && !c->ev[0]) {
+        for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
+    }
+    if (!enable) {
+        if (int rc = collect_timing(c)) return rc;
+    }
+    c->timing = enable != 0;
+    return CA_OK;
+}
+
+int ca_ctx_read_timing(ca_ctx* c, double* shared_ms, double* stream_ms, double* merge_ms,
+                       int64_t* calls, int reset) {
+    if (!c) return fail(CA_ERR_INVALID, "null context");
+    if (int rc = collect_timing(c)) return rc;
+    if (shared_ms) *shared_ms = c->phase_ms[0];
+    if (stream_ms) *stream_ms = c->phase_ms[1];
+    if (merge_ms) *merge_ms = c->phase_ms[2];
+    if (calls) *calls = c->phase_calls;
+    if (reset) {
+        c->phase_ms[0] = c->phase_ms[1] = c->phase_ms[2] = 0;
+        c->phase_calls = 0;
+    }
+    return CA_OK;
 }
 
 int ca_attn_chunks_first(ca_ctx* c, const void* q, int n_seqs, void* stream) {

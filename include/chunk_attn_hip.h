@@ -107,6 +107,15 @@ int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
  * reference's partial buffers. */
 int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
 
+/* Per-phase timing of ca_attention, measured with HIP events recorded on the stream the
+ * kernels are launched on (the reference marks the same phases with NVTX ranges,
+ * kernel_cuda.cu:1334-1433).  While enabled, every ca_attention call records four events;
+ * ca_ctx_read_timing waits for the last call and returns the accumulated milliseconds of the
+ * chunk-first launches, the sequence-first launch and the merge launch. */
+int ca_ctx_set_timing(ca_ctx* ctx, int enable);
+int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
+                       int64_t* calls, int reset);
+
 /* Numbers describing the current tables. */
 typedef struct ca_plan_info {
     int32_t n_seqs;

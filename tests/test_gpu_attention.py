@@ -1,0 +1,194 @@
+"""GPU parity: the HIP decode path, called through the C-ABI, against the CPU oracle on the
+same seeded inputs.  Tolerance atol 2e-3 / rtol 1e-2 (fp16 output, fp32 accumulation)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from chunk_attn import capi, synth
+from gpu_helpers import (ATOL, RTOL, assert_close, dev, host_state, load_workload, make_attention,
+                         oracle_output, to_dev)
+from oracle.attention_ref import textbook_attention, textbook_partials
+
+pytestmark = pytest.mark.gpu
+
+
+def rand16(rng, *shape, sigma=1.0):
+    return (rng.standard_normal(shape) * sigma).astype(np.float16)
+
+
+@pytest.mark.parametrize("c", [32, 64, 128])
+def test_two_sequences_shared_prefix(c):
+    # the reference's test_forward scenario (tests/test_chunk_attn_cpu.py:234-265) at d_head 128
+    rng = np.random.default_rng(0)
+    H = 2
+    T1, T2, P = 2 * c + 5, 2 * c + 9, 2 * c
+    k1, v1 = rand16(rng, T1, H, 128), rand16(rng, T1, H, 128)
+    k2, v2 = rand16(rng, T2, H, 128), rand16(rng, T2, H, 128)
+    k2[:P], v2[:P] = k1[:P], v1[:P]
+    attn = make_attention(H, c, 16)
+    assert attn.add_seq(list(range(T1)), to_dev(k1), to_dev(v1)) == 0
+    assert attn.add_seq(list(range(P)) + [900 + i for i in range(T2 - P)], to_dev(k2), to_dev(v2)) == 1
+    q = rand16(rng, 2, H, 128)
+    for partition in (0, 1, 2):
+        out = attn.forward(to_dev(q), partition)
+        want = np.zeros((2, H, 128))
+        for i, (k, v) in enumerate(((k1, v1), (k2, v2))):
+            for h in range(H):
+                s = k[:, h].astype(np.float64) @ q[i, h].astype(np.float64) / math.sqrt(128)
+                p = np.exp(s - s.max())
+                want[i, h] = (p / p.sum()) @ v[:, h].astype(np.float64)
+        assert_close(out, want)
+
+
+@pytest.mark.parametrize("c", [32, 64, 128])
+def test_check_result_with_textbook(c):
+    # reference tests/test_chunk_attn_cuda.py:19-72: 32 requests x 2000 tokens, 1000 shared
+    rng = np.random.default_rng(1)
+    H, B, T, P = 2, 32, 2000, 1000
+    sk, sv = rand16(rng, P, H, 128), rand16(rng, P, H, 128)
+    attn = make_attention(H, c, B * (T // c + 2))
+    for s in range(B):
+        k, v = rand16(rng, T, H, 128), rand16(rng, T, H, 128)
+        k[:P], v[:P] = sk, sv
+        toks = list(range(P)) + [100_000 * (s + 1) + i for i in range(T - P)]
+        assert attn.add_seq(toks, to_dev(k), to_dev(v)) == s
+    q = rand16(rng, B, H, 128)
+    want = oracle_output(attn, q, exact=True)
+    for partition in (0, 1, 2):
+        assert_close(attn.forward(to_dev(q), partition), want)
+    info = attn.ctx.plan_info()
+    assert info.n_seqs == B
+
+
+def test_partials_match_reference_layout():
+    # reference cpp/tests/test_gpu_kernel.cpp:8-64: 15 sequences sharing every chunk, 16 heads
+    rng = np.random.default_rng(2)
+    H, c, n, n_chunks = 16, 64, 15, 24
+    attn = make_attention(H, c, n_chunks + n + 4)
+    attn.ctx.set_plan(shared_seg_chunks=1)
+    T = n_chunks * c
+    k, v = rand16(rng, T, H, 128), rand16(rng, T, H, 128)
+    for s in range(n):
+        attn.add_seq(list(range(T)), to_dev(k), to_dev(v))
+    q = rand16(rng, n, H, 128)
+    attn.refresh_kernel_context()
+    qd = to_dev(q)
+    attn.ctx.attn_chunks_first(qd.data_ptr(), n)
+    maxs, sums, attns = attn.ctx.export_partials()
+    rows, kpool, vpool = host_state(attn)
+    ref = attn.ctx.ref_tables()
+    shared = [r for r in rows.tolist() if r[3] - r[2] > 1]
+    assert len(shared) == n_chunks == ref["n_shared"]
+    for i, (slot, nt, b, e) in enumerate(shared):
+        m, l, o = textbook_partials(q.astype(np.float32), slot, nt, b, e, kpool, vpool)
+        off, nn = int(ref["offsets"][i]), e - b
+        sl = slice(off * H, off * H + H * nn)
+        np.testing.assert_allclose(maxs[sl].reshape(H, nn), m, atol=1e-3, rtol=1e-3)
+        np.testing.assert_allclose(sums[sl].reshape(H, nn), l, atol=1e-3, rtol=2e-3)
+        np.testing.assert_allclose(attns[sl].reshape(H, nn, 128), o, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("n_shared_seqs", [1, 3, 16, 17, 40, 64, 65, 100])
+def test_any_number_of_sharing_sequences(n_shared_seqs):
+    # M tiling: row counts that are not multiples of 16 and beyond one 64-row tile
+    w = synth.prefix_workload("m-tiles", n_shared_seqs, 64, 192, 70, n_heads=4)
+    attn, order = load_workload(w)
+    assert order == list(range(w.n_seqs))
+    q = w.q()
+    assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
+
+
+def test_two_level_tree_and_remove():
+    w = synth.two_level_workload("two-level", 3, 5, 32, 96, 64, 40, n_heads=4)
+    attn, order = load_workload(w)
+    q = w.q()
+    assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
+    # removing sequences re-indexes the rest; outputs must follow
+    attn.remove_seq(7)
+    attn.remove_seq(0)
+    keep = [i for i in range(w.n_seqs) if i not in (0, 7)]
+    q2 = q[keep]
+    out = attn.forward(to_dev(q2))
+    assert_close(out, oracle_output(attn, q2))
+    assert_close(out, oracle_output(attn, q2, exact=True))
+
+
+@pytest.mark.parametrize("tpp", [0, 2, 100])
+def test_tpp_threshold(tpp):
+    w = synth.two_level_workload("tpp", 2, 3, 64, 128, 64, 30, n_heads=2)
+    attn, _ = load_workload(w, tpp_threshold=tpp)
+    q = w.q()
+    assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
+
+
+def test_append_tokens_across_chunk_boundaries():
+    c, H = 32, 4
+    w = synth.prefix_workload("append", 6, c, 64, 0, n_heads=H)
+    # ragged private parts: tails at different fill levels, one exactly full
+    lens = [1, 31, 32, 33, 5, 63]
+    for s, n in enumerate(lens):
+        w.seqs[s].append(synth.Segment(1_000_000 * (s + 1) + np.arange(n), synth.STREAM_K_UNIQUE + s, synth.STREAM_V_UNIQUE + s))
+    attn, _ = load_workload(w)
+    kv_host = [list(w.kv(s)) for s in range(w.n_seqs)]
+    rng = np.random.default_rng(3)
+    for step in range(70):
+        k, v = w.append_kv(step)
+        attn.append_token(w.append_tokens(step), to_dev(k), to_dev(v))
+        for s in range(w.n_seqs):
+            kv_host[s][0] = np.concatenate([kv_host[s][0], k[s:s + 1]])
+            kv_host[s][1] = np.concatenate([kv_host[s][1], v[s:s + 1]])
+        if step % 9 == 0 or step in (30, 31, 32, 33, 69):
+            q = rand16(rng, w.n_seqs, H, 128)
+            out = attn.forward(to_dev(q))
+            want = np.zeros((w.n_seqs, H, 128))
+            for s in range(w.n_seqs):
+                kk, vv = kv_host[s]
+                for h in range(H):
+                    sc = kk[:, h].astype(np.float64) @ q[s, h].astype(np.float64) / math.sqrt(128)
+                    p = np.exp(sc - sc.max())
+                    want[s, h] = (p / p.sum()) @ vv[:, h].astype(np.float64)
+            assert_close(out, want)
+    # the pool holds exactly the appended rows
+    rows, kpool, vpool = host_state(attn)
+    for s in range(w.n_seqs):
+        mine = [r for r in rows.tolist() if r[2] <= s < r[3]]
+        got = np.concatenate([kpool[r[0]][:, :r[1]] for r in mine if r[1]], axis=1)
+        np.testing.assert_array_equal(got, np.transpose(kv_host[s][0], (1, 0, 2)).astype(np.float32))
+
+
+def test_stale_rows_do_not_leak():
+    # a freed chunk full of NaN is reused as a partially filled tail
+    c, H = 32, 2
+    attn = make_attention(H, c, 8)
+    bad = np.full((c, H, 128), np.nan, np.float16)
+    attn.add_seq(list(range(c)), to_dev(bad), to_dev(bad))
+    attn.remove_seq(0)
+    rng = np.random.default_rng(4)
+    k, v = rand16(rng, 5, H, 128), rand16(rng, 5, H, 128)
+    attn.add_seq([7, 8, 9, 10, 11], to_dev(k), to_dev(v))
+    q = rand16(rng, 1, H, 128)
+    for partition in (0, 1, 2):
+        assert_close(attn.forward(to_dev(q), partition), oracle_output(attn, q, exact=True))
+
+
+def test_errors_through_the_c_abi():
+    attn = make_attention(2, 64, 8)
+    rng = np.random.default_rng(5)
+    k = to_dev(rand16(rng, 3, 2, 128))
+    attn.add_seq([1, 2, 3], k, k)
+    with pytest.raises(RuntimeError, match="q is not contiguous"):
+        attn.forward(to_dev(rand16(rng, 1, 2, 256))[:, :, :128])
+    with pytest.raises(capi.ChunkAttnError, match="does not match the tables"):
+        attn.forward(to_dev(rand16(rng, 2, 2, 128)))
+    with pytest.raises(RuntimeError, match="num of seqs is not equal to num of tokens"):
+        attn.append_token([1, 2], k[:2], k[:2])
+    with pytest.raises(capi.ChunkAttnError, match="Unsupported partition type"):
+        attn.forward(to_dev(rand16(rng, 1, 2, 128)), 3)
+    small = make_attention(2, 64, 0)
+    with pytest.raises(capi.ChunkAttnError, match="capacity reached"):
+        for i in range(100):
+            small.add_seq([i] * 64, to_dev(rand16(rng, 64, 2, 128)), to_dev(rand16(rng, 64, 2, 128)))
+    with pytest.raises(capi.ChunkAttnError, match="unsupported chunk_size"):
+        capi.KernelContext(2, 128, 48, 1, 1, 1)
