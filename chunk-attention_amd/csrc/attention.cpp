@@ -1,0 +1,195 @@
+#include "attention.h"
+
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPFunctions.h>
+
+#include <iostream>
+#include <stdexcept>
+
+namespace GPT {
+
+Attention::Attention(int n_heads, int d_head, int chunk_size, int memory_mb, bool share_prefix,
+                     int tpp_threshold, torch::Dtype dtype, torch::Device device)
+  : n_heads_(n_heads)
+  , d_head_(d_head)
+  , chunk_size_(chunk_size)
+  , memory_mb_(memory_mb)
+  , share_prefix_(share_prefix)
+  , tpp_threshold_(tpp_threshold)
+  , t_options_(torch::TensorOptions().dtype(dtype).layout(torch::kStrided).device(device).requires_grad(false)) {
+    init();
+}
+
+Attention::Attention(Attention& other)
+  : n_heads_(other.n_heads_)
+  , d_head_(other.d_head_)
+  , chunk_size_(other.chunk_size_)
+  , memory_mb_(other.memory_mb_)
+  , share_prefix_(other.share_prefix_)
+  , tpp_threshold_(other.tpp_threshold_)
+  , t_options_(other.t_options_) {
+    init();
+}
+
+void Attention::init() {
+    // the only kernels are HIP kernels: same check as the reference's GPU KernelContext
+    if (!t_options_.device().is_cuda()) {
+        throw std::runtime_error("GPUKernel is enabled. But the device is not CUDA.");
+    }
+    if (t_options_.dtype() != torch::kFloat16) {
+        throw std::runtime_error("unsupported data type: the HIP kernels take float16 K/V/Q");
+    }
+    if (!t_options_.device().has_index()) {
+        t_options_ = t_options_.device(torch::Device(torch::kCUDA, c10::hip::current_device()));
+    }
+    c10::DeviceGuard guard(t_options_.device());
+    max_chunks_ = ChunkAllocator::max_chunks_for(memory_mb_, chunk_size_, n_heads_, d_head_, 2);
+    const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
+    key_storage_ = torch::empty({ chunk_elems * max_chunks_ }, t_options_);
+    value_storage_ = torch::empty({ chunk_elems * max_chunks_ }, t_options_);
+    tree_ = std::make_unique<PrefixTree>(chunk_size_, max_chunks_, share_prefix_, chunk_elems * 2 * 2);
+    check(ca_ctx_create(&ctx_, n_heads_, d_head_, chunk_size_, key_storage_.data_ptr(),
+                        value_storage_.data_ptr(), max_chunks_, tpp_threshold_));
+}
+
+Attention::~Attention() { ca_ctx_destroy(ctx_); }
+
+void* Attention::stream() const {
+    return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t_options_.device().index()).stream();
+}
+
+void Attention::check(int rc) const {
+    if (rc != CA_OK) throw std::runtime_error(ca_last_error());
+}
+
+torch::Tensor Attention::checked_kv(const torch::Tensor& t, int64_t rows, const char* name) const {
+    if (t.dim() != 3 || t.size(0) != rows || t.size(1) != n_heads_ || t.size(2) != d_head_) {
+        throw std::runtime_error(std::string(name) + " must have shape [n, n_heads, d_head] with n = number of tokens");
+    }
+    if (t.scalar_type() != torch::kFloat16) throw std::runtime_error("unsupported data type");
+    if (t.device() != t_options_.device()) throw std::runtime_error(std::string(name) + " is on a different device than the cache");
+    return t.contiguous();
+}
+
+int Attention::add_seq(const std::vector<int>& tokens, torch::Tensor k, torch::Tensor v) {
+    const int n = static_cast<int>(tokens.size());
+    k = checked_kv(k, n, "k");
+    v = checked_kv(v, n, "v");
+    std::vector<CopyJob> jobs;
+    const int seq_idx = tree_->add_seq(tokens, &jobs);
+    if (!jobs.empty()) {
+        c10::DeviceGuard guard(t_options_.device());
+        std::vector<int32_t> slots;
+        slots.reserve(jobs.size());
+        for (const auto& j : jobs) slots.push_back(j.slot);
+        check(ca_scatter_kv(ctx_, k.data_ptr(), v.data_ptr(), n, jobs.front().tok_begin, slots.data(),
+                            static_cast<int>(slots.size()), stream()));
+    }
+    return seq_idx;
+}
+
+std::shared_ptr<std::future<int>> Attention::add_seq_async(const std::vector<int>&, torch::Tensor,
+                                                           torch::Tensor) {
+    // the reference's asynchronous insert is disabled the same way (attention.cpp:195-198 there)
+    throw std::runtime_error("the implementation has bugs, still have problem in capturing torch tensors in lambda");
+}
+
+void Attention::remove_seq(int seq_idx) { tree_->remove_seq(seq_idx); }
+
+void Attention::clear() { tree_->clear(); }
+
+std::vector<Chunk*> Attention::reserve() { return tree_->reserve(); }
+
+void Attention::refresh_kernel_context(bool force) {
+    if (!force && ca_ctx_valid(ctx_) && tables_version_ == tree_->version()) return;
+    c10::DeviceGuard guard(t_options_.device());
+    const auto infos = tree_->get_chunks();
+    std::vector<ca_chunk_row> rows(infos.size());
+    for (size_t i = 0; i < infos.size(); i++) {
+        rows[i] = { infos[i].chunk->slot(), infos[i].chunk->n_tokens(), infos[i].seq_idx_begin, infos[i].seq_idx_end };
+    }
+    check(ca_refresh_kernel_context(ctx_, rows.data(), static_cast<int>(rows.size()), tree_->n_seqs(), stream()));
+    tables_version_ = tree_->version();
+}
+
+std::vector<Chunk*> Attention::append_token(const std::vector<int>& tokens, torch::Tensor k,
+                                            torch::Tensor v, bool /*fused*/) {
+    if (tree_->tails().size() != tokens.size()) {
+        throw std::runtime_error("num of seqs is not equal to num of tokens");
+    }
+    const int n = static_cast<int>(tokens.size());
+    k = checked_kv(k, n, "k");
+    v = checked_kv(v, n, "v");
+    std::vector<Chunk*> fresh = tree_->reserve();
+    refresh_kernel_context();
+    {
+        c10::DeviceGuard guard(t_options_.device());
+        check(ca_append_kv(ctx_, k.data_ptr(), v.data_ptr(), n, stream()));
+    }
+    tree_->append_token_ids(tokens);
+    ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1);
+    return fresh;
+}
+
+torch::Tensor Attention::forward(torch::Tensor q, int partition) {
+    if (!q.is_contiguous()) throw std::runtime_error("q is not contiguous");
+    if (q.dim() != 3 || q.size(1) != n_heads_ || q.size(2) != d_head_) {
+        throw std::runtime_error("q must have shape [n_seqs, n_heads, d_head]");
+    }
+    if (q.scalar_type() != torch::kFloat16) throw std::runtime_error("unsupported data type");
+    if (q.device() != t_options_.device()) throw std::runtime_error("q is on a different device than the cache");
+    c10::DeviceGuard guard(t_options_.device());
+    torch::Tensor output = torch::empty({ q.size(0), n_heads_, d_head_ }, t_options_);
+    refresh_kernel_context();
+    check(ca_attention(ctx_, q.data_ptr(), output.data_ptr(), static_cast<int>(q.size(0)), partition, stream()));
+    return output;
+}
+
+void Attention::duplicate(int seq_idx, int copies) {
+    std::vector<std::pair<int, int>> pairs;
+    tree_->duplicate(seq_idx, copies, &pairs);
+    c10::DeviceGuard guard(t_options_.device());
+    for (const auto& [src, dst] : pairs) check(ca_copy_chunk(ctx_, src, dst, stream()));
+}
+
+int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::Tensor k, torch::Tensor v) {
+    // beam search step (reference attention.cpp:216-261): candidate 0 continues the sequence,
+    // candidates 1.. become copies of its tail inserted right after it, each with its own token
+    const int n = static_cast<int>(tokens.size());
+    if (n < 1) return seq_idx;
+    if (seq_idx < 0 || seq_idx >= tree_->n_seqs()) throw std::out_of_range("no such sequence");
+    k = checked_kv(k, n, "k");
+    v = checked_kv(v, n, "v");
+    tree_->reserve();
+    if (n > 1) duplicate(seq_idx, n - 1);
+    // row i of k/v becomes the next token of sequence seq_idx + i
+    c10::DeviceGuard guard(t_options_.device());
+    const auto& tails = tree_->tails();
+    for (int i = 0; i < n; i++) {
+        Chunk* tail = tails[seq_idx + i];
+        key(tail).select(1, tail->n_tokens()).copy_(k[i]);
+        value(tail).select(1, tail->n_tokens()).copy_(v[i]);
+        tail->append_tokens(tokens, i, i + 1);
+    }
+    ca_ctx_invalidate(ctx_);  // sequence lengths changed under the device tables
+    return seq_idx;
+}
+
+torch::Tensor Attention::key(const Chunk* chunk) {
+    const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
+    return key_storage_.narrow(0, chunk_elems * chunk->slot(), chunk_elems).view({ n_heads_, chunk_size_, d_head_ });
+}
+
+torch::Tensor Attention::value(const Chunk* chunk) {
+    const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
+    return value_storage_.narrow(0, chunk_elems * chunk->slot(), chunk_elems).view({ n_heads_, chunk_size_, d_head_ });
+}
+
+void Attention::print(Chunk* root, int level) {
+    if (root == nullptr) root = tree_->root();
+    std::cout << std::string(size_t(level) * 4, ' ') << root->to_string(true) << std::endl;
+    for (Chunk* child : root->children) print(child, level + 1);
+}
+
+}  // namespace GPT

@@ -131,6 +131,7 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.delta_tokens = c->delta_tokens;
     a.H = c->H;
     a.C = c->C;
+    a.d = c->d;
     a.scale_log2 = 1.4426950408889634f / std::sqrt(static_cast<float>(c->d));
     return a;
 }
@@ -225,6 +226,16 @@ int check_ready(ca_ctx* c, const void* q, int n_seqs) {
     return CA_OK;
 }
 
+// The attention kernels exist for the shapes the reference's GPU kernels take
+// (kernel_cuda.cu:1199, 1256-1265 there); like there, other shapes fail when attention is asked for.
+int check_attention_shape(const ca_ctx* c) {
+    if (c->d != 128) return fail(CA_ERR_INVALID, "unsupported head dim " + std::to_string(c->d));
+    if (c->C != 32 && c->C != 64 && c->C != 128) {
+        return fail(CA_ERR_INVALID, "unsupported chunk_size " + std::to_string(c->C));
+    }
+    return CA_OK;
+}
+
 // Adds the elapsed times of the last timed ca_attention call to the accumulators.
 int collect_timing(ca_ctx* c) {
     if (!c->ev_pending) return CA_OK;
@@ -272,11 +283,9 @@ int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k
                   void* v_pool, int max_chunks, int tpp_threshold) {
     if (!out) return fail(CA_ERR_INVALID, "null output pointer");
     *out = nullptr;
-    if (d_head != 128) return fail(CA_ERR_INVALID, "unsupported head dim " + std::to_string(d_head));
-    if (chunk_size != 32 && chunk_size != 64 && chunk_size != 128) {
-        return fail(CA_ERR_INVALID, "unsupported chunk_size " + std::to_string(chunk_size));
+    if (n_heads <= 0 || d_head <= 0 || chunk_size <= 0 || max_chunks < 0 || tpp_threshold < 0) {
+        return fail(CA_ERR_INVALID, "bad shape argument");
     }
-    if (n_heads <= 0 || max_chunks < 0 || tpp_threshold < 0) return fail(CA_ERR_INVALID, "bad shape argument");
     if (max_chunks > 0 && (!k_pool || !v_pool)) return fail(CA_ERR_INVALID, "null KV pool");
     int n_dev = 0;
     hipError_t e = hipGetDeviceCount(&n_dev);
@@ -360,6 +369,7 @@ void ca_ctx_set_delta_tokens(ca_ctx* c, int delta_tokens) {
 int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition, void* stream) {
     if (partition < 0 || partition > 2) return fail(CA_ERR_INVALID, "Unsupported partition type");
     if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
     if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
     if (n_seqs == 0) return CA_OK;
     return guarded([&]() -> int {
@@ -419,11 +429,13 @@ int ca_ctx_read_timing(ca_ctx* c, double* shared_ms, double* stream_ms, double* 
 
 int ca_attn_chunks_first(ca_ctx* c, const void* q, int n_seqs, void* stream) {
     if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
     return guarded([&]() -> int { return run_shared(c, q, static_cast<hipStream_t>(stream)); });
 }
 
 int ca_attn_seqs_first(ca_ctx* c, const void* q, void* out, int n_seqs, void* stream) {
     if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
     if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
     return guarded([&]() -> int { return run_stream_and_merge(c, q, out, static_cast<hipStream_t>(stream)); });
 }

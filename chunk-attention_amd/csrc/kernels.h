@@ -22,6 +22,7 @@ struct LaunchArgs {
     int delta_tokens = 0;
     int H = 0;
     int C = 0;
+    int d = 128;
     float scale_log2 = 0.f;  // log2(e) / sqrt(d_head)
 };
 

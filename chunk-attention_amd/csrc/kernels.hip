@@ -461,22 +461,21 @@ __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ par
 }
 
 // ---------------------------------------------------------------------------------------
-// K/V row writes.  One thread moves 16 bytes of K and of V.
+// K/V row writes.  One thread moves one piece (16 bytes when d_head allows, else 2) of K and V.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(WG) void append_kernel(const uint4* __restrict__ k,
-                                                    const uint4* __restrict__ v,
-                                                    uint4* __restrict__ kpool,
-                                                    uint4* __restrict__ vpool,
+template <typename T>
+__global__ __launch_bounds__(WG) void append_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                                    T* __restrict__ kpool, T* __restrict__ vpool,
                                                     const int32_t* __restrict__ tail_slot,
                                                     const int32_t* __restrict__ tail_fill,
-                                                    int delta_tokens, int n_seqs, int H, int C) {
-    constexpr int V16 = D / 8;  // 16-byte pieces per row
+                                                    int delta_tokens, int n_seqs, int H, int C,
+                                                    int pieces) {
     const int idx = blockIdx.x * WG + threadIdx.x;
-    if (idx >= n_seqs * H * V16) return;
-    const int piece = idx % V16, sh = idx / V16, h = sh % H, seq = sh / H;
+    if (idx >= n_seqs * H * pieces) return;
+    const int piece = idx % pieces, sh = idx / pieces, h = sh % H, seq = sh / H;
     const int row = tail_fill[seq] + delta_tokens;
     if (row >= C) return;  // host guarantees a free row; never write outside the chunk
-    const size_t dst = ((size_t(tail_slot[seq]) * H + h) * C + row) * V16 + piece;
+    const size_t dst = ((size_t(tail_slot[seq]) * H + h) * C + row) * pieces + piece;
     kpool[dst] = k[idx];
     vpool[dst] = v[idx];
 }
@@ -486,20 +485,19 @@ struct ScatterArgs {
     int32_t slots[SCATTER_SLOTS];
 };
 
-__global__ __launch_bounds__(WG) void scatter_kernel(const uint4* __restrict__ k,
-                                                     const uint4* __restrict__ v,
-                                                     uint4* __restrict__ kpool,
-                                                     uint4* __restrict__ vpool, ScatterArgs args,
-                                                     int tok_begin, int n_copy, int H, int C) {
-    constexpr int V16 = D / 8;
+template <typename T>
+__global__ __launch_bounds__(WG) void scatter_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                                     T* __restrict__ kpool, T* __restrict__ vpool,
+                                                     ScatterArgs args, int tok_begin, int n_copy,
+                                                     int H, int C, int pieces) {
     const int64_t idx = int64_t(blockIdx.x) * WG + threadIdx.x;
-    if (idx >= int64_t(n_copy) * H * V16) return;
-    const int piece = idx % V16;
-    const int h = (idx / V16) % H;
-    const int t = idx / (int64_t(V16) * H);  // token within this launch
+    if (idx >= int64_t(n_copy) * H * pieces) return;
+    const int piece = idx % pieces;
+    const int h = (idx / pieces) % H;
+    const int t = idx / (int64_t(pieces) * H);  // token within this launch
     const int slot = args.slots[t / C];
-    const size_t dst = ((size_t(slot) * H + h) * C + (t % C)) * V16 + piece;
-    const size_t src = (size_t(tok_begin + t) * H + h) * V16 + piece;
+    const size_t dst = ((size_t(slot) * H + h) * C + (t % C)) * pieces + piece;
+    const size_t src = (size_t(tok_begin + t) * H + h) * pieces + piece;
     kpool[dst] = k[src];
     vpool[dst] = v[src];
 }
@@ -592,18 +590,29 @@ int launch_merge(const LaunchArgs& a, const int32_t* part_ptr, const int32_t* pa
 int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32_t* tail_slot,
                   const int32_t* tail_fill, int n_seqs, hipStream_t st) {
     if (n_seqs <= 0) return 0;
-    const int total = n_seqs * a.H * (D / 8);
-    hipLaunchKernelGGL(append_kernel, dim3((total + WG - 1) / WG), dim3(WG), 0, st,
-                       static_cast<const uint4*>(k), static_cast<const uint4*>(v),
-                       static_cast<uint4*>(const_cast<void*>(a.kpool)),
-                       static_cast<uint4*>(const_cast<void*>(a.vpool)), tail_slot, tail_fill,
-                       a.delta_tokens, n_seqs, a.H, a.C);
+    void* kp = const_cast<void*>(a.kpool);
+    void* vp = const_cast<void*>(a.vpool);
+    if (a.d % 8 == 0) {
+        const int pieces = a.d / 8, total = n_seqs * a.H * pieces;
+        hipLaunchKernelGGL(append_kernel<uint4>, dim3((total + WG - 1) / WG), dim3(WG), 0, st,
+                           static_cast<const uint4*>(k), static_cast<const uint4*>(v),
+                           static_cast<uint4*>(kp), static_cast<uint4*>(vp), tail_slot, tail_fill,
+                           a.delta_tokens, n_seqs, a.H, a.C, pieces);
+    } else {
+        const int pieces = a.d, total = n_seqs * a.H * pieces;
+        hipLaunchKernelGGL(append_kernel<uint16_t>, dim3((total + WG - 1) / WG), dim3(WG), 0, st,
+                           static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v),
+                           static_cast<uint16_t*>(kp), static_cast<uint16_t*>(vp), tail_slot,
+                           tail_fill, a.delta_tokens, n_seqs, a.H, a.C, pieces);
+    }
     CA_LAUNCH_CHECK();
     return 0;
 }
 
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,
                    const int32_t* slots, int n_slots, hipStream_t st) {
+    void* kp = const_cast<void*>(a.kpool);
+    void* vp = const_cast<void*>(a.vpool);
     for (int s0 = 0; s0 < n_slots; s0 += SCATTER_SLOTS) {
         const int ns = (n_slots - s0 < SCATTER_SLOTS) ? (n_slots - s0) : SCATTER_SLOTS;
         const int t0 = tok_begin + s0 * a.C;
@@ -612,13 +621,21 @@ int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_toke
         if (n_copy <= 0) break;
         ScatterArgs args;
         for (int i = 0; i < SCATTER_SLOTS; i++) args.slots[i] = (i < ns) ? slots[s0 + i] : 0;
-        const int64_t total = int64_t(n_copy) * a.H * (D / 8);
-        hipLaunchKernelGGL(scatter_kernel, dim3(static_cast<unsigned>((total + WG - 1) / WG)),
-                           dim3(WG), 0, st, static_cast<const uint4*>(k),
-                           static_cast<const uint4*>(v),
-                           static_cast<uint4*>(const_cast<void*>(a.kpool)),
-                           static_cast<uint4*>(const_cast<void*>(a.vpool)), args, t0, n_copy, a.H,
-                           a.C);
+        if (a.d % 8 == 0) {
+            const int pieces = a.d / 8;
+            const int64_t total = int64_t(n_copy) * a.H * pieces;
+            hipLaunchKernelGGL(scatter_kernel<uint4>, dim3(static_cast<unsigned>((total + WG - 1) / WG)),
+                               dim3(WG), 0, st, static_cast<const uint4*>(k), static_cast<const uint4*>(v),
+                               static_cast<uint4*>(kp), static_cast<uint4*>(vp), args, t0, n_copy, a.H,
+                               a.C, pieces);
+        } else {
+            const int pieces = a.d;
+            const int64_t total = int64_t(n_copy) * a.H * pieces;
+            hipLaunchKernelGGL(scatter_kernel<uint16_t>, dim3(static_cast<unsigned>((total + WG - 1) / WG)),
+                               dim3(WG), 0, st, static_cast<const uint16_t*>(k),
+                               static_cast<const uint16_t*>(v), static_cast<uint16_t*>(kp),
+                               static_cast<uint16_t*>(vp), args, t0, n_copy, a.H, a.C, pieces);
+        }
         CA_LAUNCH_CHECK();
     }
     return 0;

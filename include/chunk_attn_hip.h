@@ -53,8 +53,9 @@ typedef struct ca_chunk_row {
     int32_t seq_end;
 } ca_chunk_row;
 
-/* Replaces KernelContext's constructor (kernel_cuda.h:10-31).  d_head must be 128 and
- * chunk_size one of 32, 64, 128, as in the reference (kernel_cuda.cu:1199, 1256-1265).
+/* Replaces KernelContext's constructor (kernel_cuda.h:10-31).  Any shape is accepted here;
+ * the attention entry points need d_head 128 and chunk_size 32, 64 or 128 and fail with
+ * CA_ERR_INVALID otherwise, as the reference's do (kernel_cuda.cu:1199, 1256-1265).
  * The pools stay owned by the caller and must outlive the context. */
 int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k_pool,
                   void* v_pool, int max_chunks, int tpp_threshold);

@@ -33,5 +33,5 @@ def test_device_entry_points_fail_loudly_without_a_gpu():
         capi.KernelContext(2, 128, 64, 0, 0, 0)
     assert "no HIP device" in str(e.value)
     h = ctypes.c_void_p()
-    assert capi.load().ca_ctx_create(ctypes.byref(h), 2, 64, 64, None, None, 0, 1) == -1   # d_head 64
-    assert b"unsupported head dim" in capi.load().ca_last_error()
+    assert capi.load().ca_ctx_create(ctypes.byref(h), 0, 64, 64, None, None, 0, 1) == -1
+    assert b"bad shape" in capi.load().ca_last_error()

@@ -190,5 +190,7 @@ def test_errors_through_the_c_abi():
     with pytest.raises(capi.ChunkAttnError, match="capacity reached"):
         for i in range(100):
             small.add_seq([i] * 64, to_dev(rand16(rng, 64, 2, 128)), to_dev(rand16(rng, 64, 2, 128)))
-    with pytest.raises(capi.ChunkAttnError, match="unsupported chunk_size"):
-        capi.KernelContext(2, 128, 48, 1, 1, 1)
+    odd = capi.Attention(n_heads=2, d_head=128, chunk_size=48, memory_mb=4, dtype=torch.float16, device=dev())
+    odd.add_seq([1, 2, 3], k, k)
+    with pytest.raises(capi.ChunkAttnError, match="unsupported chunk_size 48"):
+        odd.forward(to_dev(rand16(rng, 1, 2, 128)))
