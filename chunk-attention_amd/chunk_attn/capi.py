@@ -16,7 +16,8 @@ from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libchunkattn_hip.so")
+_LIB_PATH = os.environ.get("CHUNK_ATTN_HIP_LIB") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", "libchunkattn_hip.so")
 _lib = None
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
@@ -70,6 +71,7 @@ SIGNATURES = {
     "ca_ctx_ref_tables": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
     "ca_ctx_export_partials": (ctypes.c_int, [ctypes.c_void_p, c_f32_p, c_f32_p, c_f32_p,
                                               ctypes.c_void_p]),
+    "ca_ctx_read_partials_raw": (ctypes.c_int, [ctypes.c_void_p, c_f32_p, ctypes.c_int64, ctypes.c_void_p]),
     "ca_tables_build": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ChunkRow)] +
                         [ctypes.c_int] * 9),
     "ca_tables_destroy": (None, [ctypes.c_void_p]),
@@ -345,8 +347,9 @@ class KernelContext:
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
 
-    def set_timing(self, enable: bool) -> None:
-        _check(self._lib.ca_ctx_set_timing(self._h, int(enable)))
+    def set_timing(self, mode: int) -> None:
+        """0 off, 1 time the fused launch, 2 run and time the three phases separately."""
+        _check(self._lib.ca_ctx_set_timing(self._h, int(mode)))
 
     def read_timing(self, reset: bool = True) -> dict:
         """Accumulated per-phase milliseconds of the timed ca_attention calls."""
@@ -377,6 +380,13 @@ class KernelContext:
         t["n_shared"] = info.n_shared_chunks
         t["partial_rows"] = info.ref_partial_rows
         return t
+
+    def read_partials_raw(self, stream: int = 0) -> np.ndarray:
+        """[n_part_rows, n_heads, 160] float32 copy of the partial-row buffer."""
+        info = self.plan_info()
+        out = np.zeros((info.n_part_rows, self.n_heads, 160), np.float32)
+        _check(self._lib.ca_ctx_read_partials_raw(self._h, out.ctypes.data_as(c_f32_p), out.size, stream))
+        return out
 
     def export_partials(self, stream: int = 0):
         """(maxs, sums [rows*H], attns [rows*H, d]) in the reference's partial layout."""

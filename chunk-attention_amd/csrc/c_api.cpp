@@ -58,8 +58,6 @@ int guarded(F&& f) {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-int mb_class(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4); }
-
 }  // namespace
 
 // ---- kernel context ------------------------------------------------------------------------
@@ -93,13 +91,15 @@ struct ca_ctx {
     // offsets into dev_blob
     size_t off_shared = 0, off_stream = 0, off_slots = 0, off_seq_len = 0, off_part_ptr = 0,
            off_part_rows = 0, off_tail_slot = 0, off_tail_fill = 0;
-    int n_shared_mb[3] = { 0, 0, 0 };  // items per 16-row-block class (1, 2, 4), stored in that order
 
     float* part = nullptr;
     size_t part_cap = 0;  // bytes
+    int32_t* counters = nullptr;  // [n_seqs * H] partials finished per (sequence, head)
+    size_t counters_cap = 0;      // bytes
 
-    // optional per-phase timing: events recorded on the caller's stream around the launches
-    bool timing = false;
+    // optional timing: events recorded on the caller's stream around the launches.
+    // 1: the fused launch; 2: forward run as three timed launches (chunk-first, sequence-first, merge)
+    int timing = 0;
     hipEvent_t ev[4] = { nullptr, nullptr, nullptr, nullptr };
     bool ev_pending = false;
     double phase_ms[3] = { 0, 0, 0 };
@@ -126,8 +126,13 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.kpool = c->k_pool;
     a.vpool = c->v_pool;
     a.part = c->part;
+    a.shared_items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_shared);
+    a.stream_items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream);
     a.slots = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_slots);
     a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
+    a.part_ptr = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr);
+    a.part_rows = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows);
+    a.counters = c->counters;
     a.delta_tokens = c->delta_tokens;
     a.H = c->H;
     a.C = c->C;
@@ -153,17 +158,6 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     pp.n_cus = c->n_cus;
     ca::build_plan(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, pp, &c->plan);
     ca::Plan& p = c->plan;
-
-    // shared items grouped by how many 16-row blocks they need
-    std::stable_sort(p.shared_items.begin(), p.shared_items.end(),
-                     [](const ca::WorkItem& a, const ca::WorkItem& b) {
-                         return mb_class(a.n_rows) < mb_class(b.n_rows);
-                     });
-    c->n_shared_mb[0] = c->n_shared_mb[1] = c->n_shared_mb[2] = 0;
-    for (const auto& it : p.shared_items) {
-        const int mb = mb_class(it.n_rows);
-        c->n_shared_mb[mb == 1 ? 0 : (mb == 2 ? 1 : 2)]++;
-    }
 
     size_t off = 0;
     auto place = [&](size_t bytes) {
@@ -211,6 +205,10 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
 
     const size_t part_bytes = std::max<size_t>(size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4, 256);
     if (int rc = ensure_dev(reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
+    // completion counters start at zero; each forward leaves them at zero again
+    const int n_counters = std::max(c->n_seqs * c->H, 1);
+    if (int rc = ensure_dev(reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
+    if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
     c->partition = partition;
     return CA_OK;
 }
@@ -252,25 +250,27 @@ int collect_timing(ca_ctx* c) {
 
 int run_shared(ca_ctx* c, const void* q, hipStream_t st) {
     const ca::LaunchArgs a = launch_args(c, q, nullptr);
-    const ca::WorkItem* items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_shared);
-    const int mbs[3] = { 1, 2, 4 };
-    for (int k = 0; k < 3; k++) {
-        if (int rc = launch_rc(ca::launch_shared(a, items, c->n_shared_mb[k], mbs[k], st), "chunk-first launch")) return rc;
-        items += c->n_shared_mb[k];
-    }
-    return CA_OK;
+    return launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()), 0, false, st),
+                     "chunk-first launch");
 }
 
-int run_stream_and_merge(ca_ctx* c, const void* q, void* out, hipStream_t st) {
+int run_stream(ca_ctx* c, const void* q, void* out, hipStream_t st) {
     const ca::LaunchArgs a = launch_args(c, q, out);
-    const ca::WorkItem* items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream);
-    if (int rc = launch_rc(ca::launch_stream(a, items, static_cast<int>(c->plan.stream_items.size()), st), "sequence-first launch")) return rc;
-    if (!c->plan.part_rows.empty()) {
-        if (int rc = launch_rc(ca::launch_merge(a, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr),
-                                                reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows),
-                                                c->n_seqs, st), "merge launch")) return rc;
-    }
-    return CA_OK;
+    return launch_rc(ca::launch_decode(a, 0, static_cast<int>(c->plan.stream_items.size()), false, st),
+                     "sequence-first launch");
+}
+
+int run_merge(ca_ctx* c, void* out, hipStream_t st) {
+    if (c->plan.part_rows.empty()) return CA_OK;
+    const ca::LaunchArgs a = launch_args(c, nullptr, out);
+    return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
+}
+
+int run_fused(ca_ctx* c, const void* q, void* out, hipStream_t st) {
+    const ca::LaunchArgs a = launch_args(c, q, out);
+    return launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                       static_cast<int>(c->plan.stream_items.size()), true, st),
+                     "decode launch");
 }
 
 }  // namespace
@@ -321,6 +321,7 @@ void ca_ctx_destroy(ca_ctx* c) {
     if (!c) return;
     if (c->dev_blob) (void)hipFree(c->dev_blob);
     if (c->part) (void)hipFree(c->part);
+    if (c->counters) (void)hipFree(c->counters);
     for (int i = 0; i < 2; i++) {
         if (c->host_blob_free[i]) {
             (void)hipEventSynchronize(c->host_blob_free[i]);
@@ -377,22 +378,19 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
         if (partition != c->partition) {
             if (int rc = build_and_upload(c, partition, st)) return rc;
         }
-        if (!c->timing) {
-            if (int rc = run_shared(c, q, st)) return rc;
-            return run_stream_and_merge(c, q, out, st);
-        }
+        if (!c->timing) return run_fused(c, q, out, st);
         if (int rc = collect_timing(c)) return rc;
-        const ca::LaunchArgs a = launch_args(c, q, out);
         CA_HIP(hipEventRecord(c->ev[0], st));
-        if (int rc = run_shared(c, q, st)) return rc;
-        CA_HIP(hipEventRecord(c->ev[1], st));
-        if (int rc = launch_rc(ca::launch_stream(a, reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream),
-                                                 static_cast<int>(c->plan.stream_items.size()), st), "sequence-first launch")) return rc;
-        CA_HIP(hipEventRecord(c->ev[2], st));
-        if (!c->plan.part_rows.empty()) {
-            if (int rc = launch_rc(ca::launch_merge(a, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr),
-                                                    reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows),
-                                                    c->n_seqs, st), "merge launch")) return rc;
+        if (c->timing == 1) {
+            if (int rc = run_fused(c, q, out, st)) return rc;
+            CA_HIP(hipEventRecord(c->ev[1], st));
+            CA_HIP(hipEventRecord(c->ev[2], st));
+        } else {
+            if (int rc = run_shared(c, q, st)) return rc;
+            CA_HIP(hipEventRecord(c->ev[1], st));
+            if (int rc = run_stream(c, q, out, st)) return rc;
+            CA_HIP(hipEventRecord(c->ev[2], st));
+            if (int rc = run_merge(c, out, st)) return rc;
         }
         CA_HIP(hipEventRecord(c->ev[3], st));
         c->ev_pending = true;
@@ -405,10 +403,9 @@ int ca_ctx_set_timing(ca_ctx* c, int enable) {
     if (enable && !c->ev[0]) {
         for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
     }
-    if (!enable) {
-        if (int rc = collect_timing(c)) return rc;
-    }
-    c->timing = enable != 0;
+    if (enable < 0 || enable > 2) return fail(CA_ERR_INVALID, "timing mode must be 0, 1 or 2");
+    if (int rc = collect_timing(c)) return rc;
+    c->timing = enable;
     return CA_OK;
 }
 
@@ -437,7 +434,10 @@ int ca_attn_seqs_first(ca_ctx* c, const void* q, void* out, int n_seqs, void* st
     if (int rc = check_ready(c, q, n_seqs)) return rc;
     if (int rc = check_attention_shape(c)) return rc;
     if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
-    return guarded([&]() -> int { return run_stream_and_merge(c, q, out, static_cast<hipStream_t>(stream)); });
+    return guarded([&]() -> int {
+        if (int rc = run_stream(c, q, out, static_cast<hipStream_t>(stream))) return rc;
+        return run_merge(c, out, static_cast<hipStream_t>(stream));
+    });
 }
 
 int ca_append_kv(ca_ctx* c, const void* k, const void* v, int n_seqs, void* stream) {
@@ -556,6 +556,16 @@ int ca_ctx_export_partials(ca_ctx* c, float* maxs, float* sums, float* attns, vo
         }
         return CA_OK;
     });
+}
+
+int ca_ctx_read_partials_raw(ca_ctx* c, float* out, int64_t n_floats, void* stream) {
+    if (!c || !out || n_floats < 0) return fail(CA_ERR_INVALID, "bad argument");
+    const int64_t have = int64_t(c->plan.n_part_rows) * c->H * ca::PART_STRIDE;
+    const int64_t n = std::min(n_floats, have);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n > 0) CA_HIP(hipMemcpyAsync(out, c->part, size_t(n) * 4, hipMemcpyDeviceToHost, st));
+    CA_HIP(hipStreamSynchronize(st));
+    return CA_OK;
 }
 
 // ---- host-only table builder ---------------------------------------------------------------

@@ -9,7 +9,7 @@
 
 namespace ca {
 
-constexpr int PART_STRIDE = 132;  // floats per partial row: max, sum, 2 pad, 128 acc
+constexpr int PART_STRIDE = 160;  // floats per partial row: max, sum, 2 pad, 128 acc, pad to 5 x 128 B
 
 struct LaunchArgs {
     const void* q = nullptr;      // [n_seqs, H, 128] fp16
@@ -17,8 +17,13 @@ struct LaunchArgs {
     const void* kpool = nullptr;  // [max_chunks, H, C, 128] fp16
     const void* vpool = nullptr;
     float* part = nullptr;        // [n_part_rows, H, PART_STRIDE]
+    const WorkItem* shared_items = nullptr;
+    const WorkItem* stream_items = nullptr;
     const int32_t* slots = nullptr;
     const int32_t* seq_len = nullptr;
+    const int32_t* part_ptr = nullptr;
+    const int32_t* part_rows = nullptr;
+    int32_t* counters = nullptr;  // [n_seqs * H], zero between launches
     int delta_tokens = 0;
     int H = 0;
     int C = 0;
@@ -27,11 +32,13 @@ struct LaunchArgs {
 };
 
 // All return 0, -1 for an unsupported shape, or a positive hipError_t.
-int launch_stream(const LaunchArgs& a, const WorkItem* items, int n_items, hipStream_t st);
-// mb: 16-row blocks per item (1, 2 or 4); every item of the launch has n_rows <= 16*mb
-int launch_shared(const LaunchArgs& a, const WorkItem* items, int n_items, int mb, hipStream_t st);
-int launch_merge(const LaunchArgs& a, const int32_t* part_ptr, const int32_t* part_rows,
-                 int n_seqs, hipStream_t st);
+// One launch over the first n_shared_items shared items and the first n_stream_items stream
+// items.  fuse_merge: the workgroup finishing the last partial of a (sequence, head) writes
+// its output; otherwise only partial rows (and direct outputs) are written.
+int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, bool fuse_merge,
+                  hipStream_t st);
+int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st);
+int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st);
 int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32_t* tail_slot,
                   const int32_t* tail_fill, int n_seqs, hipStream_t st);
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,

@@ -1,16 +1,21 @@
 // HIP kernels of the ChunkAttention decode path for gfx950 (MI355X), fp16 K/V/Q, d_head 128.
 //
-//   shared_kernel   chunk-first phase: one workgroup attends a segment of shared chunks for up
-//                   to 64 sequences at once on the matrix cores (S^T = K.Q^T, O^T = V^T.P^T)
-//                   and writes one partial (max, sum, acc) row per sequence.
-//   stream_kernel   sequence-first phase: one workgroup streams a run of one sequence's own
-//                   chunks at HBM speed (16-byte coalesced loads, fp32 online softmax) and
-//                   writes one partial row, or the final output when nothing else is merged.
-//   merge_kernel    combines the partial rows of every (sequence, head) and normalises.
+//   decode_kernel   one launch for a whole forward.  Its first workgroups run the chunk-first
+//                   phase (shared_path): a segment of shared chunks is attended for up to 32
+//                   sequences at once on the matrix cores (S^T = K.Q^T, O^T = V^T.P^T), one
+//                   partial (max, sum, acc) row per sequence.  The others run the sequence-
+//                   first phase (stream_path): a run of one sequence's own chunks is streamed
+//                   at HBM speed (16-byte coalesced loads, fp32 online softmax) into one
+//                   partial row, or straight into the output when nothing else is merged.
+//                   The workgroup that completes the last partial of a (sequence, head)
+//                   merges them and writes the normalised output.
+//   merge_kernel    the same merge as a launch of its own, for the two-call
+//                   chunks-first / sequences-first interface.
 //   append_kernel / scatter_kernel   K/V row writes into the chunk pool.
 //
 // Partial rows live in base-2 units: max holds score*log2(e)/sqrt(d), sums and acc are
-// relative to 2^max.  Row layout: [0] max, [1] sum, [4..131] acc (fp32).
+// relative to 2^max.  Row layout: [0] max, [1] sum, [4..131] acc (fp32); rows are 640 B apart so
+// that no 128-byte line holds data of two writers.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -45,6 +50,27 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Partial rows are written by one workgroup and read by another, possibly on a different XCD
+// whose L2 is not coherent with the writer's.  They are therefore moved with device-scope
+// relaxed atomics (write-through stores, L2-bypassing loads): no cache-wide fence is needed,
+// only "stores done" (a workgroup barrier) before the completion counter is bumped.
+__device__ __forceinline__ void part_store(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void part_store2(float* p, float a, float b) {
+    union { f2 f; uint64_t u; } x;
+    x.f = f2{ a, b };
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float part_load(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f2 part_load2(const float* p) {
+    union { f2 f; uint64_t u; } x;
+    x.u = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return x.f;
+}
 
 __device__ __forceinline__ float dot8(const h8& a, const h8& b, float acc) {
     acc = __builtin_amdgcn_fdot2(h2{ a[0], a[1] }, h2{ b[0], b[1] }, acc, false);
@@ -106,26 +132,108 @@ __device__ __forceinline__ float reduce_rows16(float (&v)[NV], int j) {
 // Lane l = 16*g + j reads, for load i, the 16 bytes at offset 1024*i + 16*l of a sub-tile:
 // row 4*i + g, dims 8*j..8*j+7, so every load instruction covers 1 KiB of contiguous memory.
 // ---------------------------------------------------------------------------------------
+// Everything a workgroup needs besides its work item.
+struct DecodeArgs {
+    const half_t* q;
+    const half_t* kpool;
+    const half_t* vpool;
+    half_t* out;
+    float* part;
+    const WorkItem* shared_items;
+    const WorkItem* stream_items;
+    const int32_t* slots;
+    const int32_t* seq_len;
+    const int32_t* part_ptr;
+    const int32_t* part_rows;
+    int32_t* counters;  // [n_seqs * H] partial rows completed so far, 0 between launches
+    int n_shared_wgs;   // workgroups [0, n_shared_wgs) run shared items
+    int delta_tokens;
+    int H;
+    float scale_log2;
+    int fuse_merge;  // 1: the last workgroup to finish a (sequence, head) merges its partials
+};
+
+// Wave-level merge of the partial rows of one (sequence, head): lane l owns output dims
+// 2l, 2l+1.  Maxima and sums are fetched 64 rows at a time, one per lane; the acc rows are
+// then read with independent loads.
+__device__ __forceinline__ void merge_rows(const float* __restrict__ part,
+                                           const int32_t* __restrict__ part_rows, int p0, int p1,
+                                           int h, int H, half_t* __restrict__ out_row, int l) {
+    float m = NEG_INF;
+    for (int p = p0 + l; p < p1; p += 64) {
+        m = fmaxf(m, part_load(part + (size_t(part_rows[p]) * H + h) * PART_STRIDE));
+    }
+    m = wave_max(m);
+    float lsum = 0.f;
+    f2 o = f2{ 0.f, 0.f };
+    for (int pb = p0; pb < p1; pb += 64) {
+        float wp = 0.f;
+        int rowp = 0;
+        if (pb + l < p1) {
+            rowp = part_rows[pb + l];
+            const float* r = part + (size_t(rowp) * H + h) * PART_STRIDE;
+            const float mp = part_load(r);
+            wp = (mp == NEG_INF) ? 0.f : fast_exp2(mp - m);
+            lsum += wp * part_load(r + 1);
+        }
+        const int cnt = (p1 - pb < 64) ? (p1 - pb) : 64;
+#pragma unroll 8
+        for (int k = 0; k < cnt; k++) {
+            const float wk = __shfl(wp, k, 64);
+            const int rk = __shfl(rowp, k, 64);
+            const f2 v = part_load2(part + (size_t(rk) * H + h) * PART_STRIDE + 4 + 2 * l);
+            o += wk * v;
+        }
+    }
+    lsum = wave_sum(lsum);
+    const float r = lsum > 0.f ? 1.f / lsum : 0.f;
+    *reinterpret_cast<h2*>(out_row + 2 * l) = h2{ half_t(o[0] * r), half_t(o[1] * r) };
+}
+
+// LDS of one workgroup, shared by the two paths.
+constexpr int VPITCH = D + 4;  // halves per LDS row of a V block: 264 B keeps the four token
+                               // groups on disjoint banks for 2-byte column reads
+constexpr int OPITCH = D + 4;  // floats per row of the cross-wave accumulation buffer
+constexpr int MB = 2;          // 16-row blocks per shared item
+constexpr int MROWS = 16 * MB;
+struct SharedPathLds {
+    half_t v[NW][16 * VPITCH];
+    float o[MROWS * OPITCH];
+    float m[NW][MROWS];
+    float l[NW][MROWS];
+    int last[MROWS];
+};
+struct StreamPathLds {
+    float p[NW][64];
+    float o[NW][D];
+    float m[NW];
+    float l[NW];
+    float own_o[D];  // the workgroup's combined result, kept for the in-place merge
+    float own_m, own_l;
+    int state;       // 0: not last, 1: last after publishing the partial, 2: last without publishing
+};
+union __attribute__((aligned(16))) DecodeLds {
+    SharedPathLds sh;
+    StreamPathLds st;
+};
+
 template <int C>
-__global__ __launch_bounds__(WG) void stream_kernel(
-  const half_t* __restrict__ q, const half_t* __restrict__ kpool,
-  const half_t* __restrict__ vpool, half_t* __restrict__ out, float* __restrict__ part,
-  const WorkItem* __restrict__ items, const int32_t* __restrict__ slots,
-  const int32_t* __restrict__ seq_len, int delta_tokens, int H, float scale_log2) {
+__device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem& it, int h,
+                                            StreamPathLds& sm) {
+    const half_t* __restrict__ q = A.q;
+    const half_t* __restrict__ kpool = A.kpool;
+    const half_t* __restrict__ vpool = A.vpool;
+    const int32_t* __restrict__ slots = A.slots;
+    const int H = A.H;
+    const float scale_log2 = A.scale_log2;
     constexpr int SUB = (C < 64) ? C : 64;  // tokens per sub-tile
     constexpr int NL = SUB / 4;             // 16-byte loads per lane per sub-tile
     constexpr int NSUB = C / SUB;
 
-    const int h = blockIdx.x % H;
-    const WorkItem it = items[blockIdx.x / H];
     const int tid = threadIdx.x;
     const int w = tid >> 6, l = tid & 63, g = l >> 4, j = l & 15;
     const int seq = it.seq_begin;
-    const int len = seq_len[it.len_seq] + delta_tokens;
-
-    __shared__ float sm_p[NW][64];
-    __shared__ float sm_o[NW][D];
-    __shared__ float sm_m[NW], sm_l[NW];
+    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
 
     const h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
 
@@ -176,14 +284,14 @@ __global__ __launch_bounds__(WG) void stream_kernel(
             const float p = fast_exp2(s - m_new);
             m_run = m_new;
             l_lane = l_lane * alpha + p;
-            sm_p[w][l] = p;
+            sm.p[w][l] = p;
 #pragma unroll
             for (int e = 0; e < 8; e++) acc[e] *= alpha;
             __builtin_amdgcn_wave_barrier();
             float pr[NL];
 #pragma unroll
             for (int i = 0; i < NL; i += 4) {
-                const f4 t4 = *reinterpret_cast<const f4*>(&sm_p[w][16 * g + i]);
+                const f4 t4 = *reinterpret_cast<const f4*>(&sm.p[w][16 * g + i]);
                 pr[i] = t4[0]; pr[i + 1] = t4[1]; pr[i + 2] = t4[2]; pr[i + 3] = t4[3];
             }
             __builtin_amdgcn_wave_barrier();
@@ -205,44 +313,117 @@ __global__ __launch_bounds__(WG) void stream_kernel(
     }
     if (g == 0) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) sm_o[w][8 * j + e] = acc[e];
+        for (int e = 0; e < 8; e++) sm.o[w][8 * j + e] = acc[e];
     }
     if (l == 0) {
-        sm_m[w] = m_run;
-        sm_l[w] = l_wave;
+        sm.m[w] = m_run;
+        sm.l[w] = l_wave;
     }
     __syncthreads();
 
-    if (tid < D) {
-        float m = sm_m[0];
+    // combine the four waves: thread tid < 128 owns output dim tid
+    float m = sm.m[0];
 #pragma unroll
-        for (int k = 1; k < NW; k++) m = fmaxf(m, sm_m[k]);
-        float o = 0.f, lsum = 0.f;
+    for (int k = 1; k < NW; k++) m = fmaxf(m, sm.m[k]);
+    float o = 0.f, lsum = 0.f;
+    if (tid < D) {
 #pragma unroll
         for (int k = 0; k < NW; k++) {
-            const float f = (sm_m[k] == NEG_INF) ? 0.f : fast_exp2(sm_m[k] - m);
-            o += f * sm_o[k][tid];
-            lsum += f * sm_l[k];
+            const float f = (sm.m[k] == NEG_INF) ? 0.f : fast_exp2(sm.m[k] - m);
+            o += f * sm.o[k][tid];
+            lsum += f * sm.l[k];
         }
-        if (it.part_row >= 0) {
-            float* row = part + (size_t(it.part_row) * H + h) * PART_STRIDE;
-            row[4 + tid] = o;
-            if (tid == 0) {
-                row[0] = m;
-                row[1] = lsum;
-            }
-        } else {
+    }
+    if (it.part_row < 0) {  // nothing else to merge: final output
+        if (tid < D) {
             const float r = lsum > 0.f ? 1.f / lsum : 0.f;
-            out[(size_t(seq) * H + h) * D + tid] = half_t(o * r);
+            A.out[(size_t(seq) * H + h) * D + tid] = half_t(o * r);
         }
+        return;
+    }
+    float* own_row = A.part + (size_t(it.part_row) * H + h) * PART_STRIDE;
+    if (!A.fuse_merge) {
+        if (tid < D) part_store(own_row + 4 + tid, o);
+        if (tid == 0) part_store2(own_row, m, lsum);
+        return;
+    }
+
+    // Fused merge.  If every other partial of this (sequence, head) is already complete, merge
+    // straight from LDS without publishing this one; otherwise publish, count, and let whoever
+    // arrives last merge from memory.
+    const int p0 = A.part_ptr[seq], p1 = A.part_ptr[seq + 1];
+    int* counter = &A.counters[seq * H + h];
+    if (tid == 0) {
+        sm.state = (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p1 - p0 - 1) ? 2 : 0;
+    }
+    if (tid < D) sm.own_o[tid] = o;
+    if (tid == 0) {
+        sm.own_m = m;
+        sm.own_l = lsum;
+    }
+    __syncthreads();
+    if (sm.state == 2) {
+        // wave w folds partial rows w, w+4, ... (not our own) into a running (m, l, acc)
+        float mw = NEG_INF, lw = 0.f;
+        f2 ow = f2{ 0.f, 0.f };
+        for (int p = p0 + w; p < p1; p += NW) {
+            const int row = A.part_rows[p];
+            if (row == it.part_row) continue;
+            const float* r = A.part + (size_t(row) * H + h) * PART_STRIDE;
+            const f2 ml = part_load2(r);
+            const f2 v = part_load2(r + 4 + 2 * l);
+            const float mn = fmaxf(mw, ml[0]);
+            const float fa = (mw == NEG_INF) ? 0.f : fast_exp2(mw - mn);
+            const float fb = (ml[0] == NEG_INF) ? 0.f : fast_exp2(ml[0] - mn);
+            ow = fa * ow + fb * v;
+            lw = fa * lw + fb * ml[1];
+            mw = mn;
+        }
+        __syncthreads();  // everyone has read sm.o / sm.m / sm.l of the first combine
+        sm.o[w][2 * l] = ow[0];
+        sm.o[w][2 * l + 1] = ow[1];
+        if (l == 0) {
+            sm.m[w] = mw;
+            sm.l[w] = lw;
+        }
+        __syncthreads();
+        if (tid < D) {
+            float mm = sm.own_m;
+#pragma unroll
+            for (int k = 0; k < NW; k++) mm = fmaxf(mm, sm.m[k]);
+            const float f0 = (sm.own_m == NEG_INF) ? 0.f : fast_exp2(sm.own_m - mm);
+            float oo = f0 * sm.own_o[tid], ll = f0 * sm.own_l;
+#pragma unroll
+            for (int k = 0; k < NW; k++) {
+                const float f = (sm.m[k] == NEG_INF) ? 0.f : fast_exp2(sm.m[k] - mm);
+                oo += f * sm.o[k][tid];
+                ll += f * sm.l[k];
+            }
+            const float r = ll > 0.f ? 1.f / ll : 0.f;
+            A.out[(size_t(seq) * H + h) * D + tid] = half_t(oo * r);
+        }
+        if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    if (tid < D) part_store(own_row + 4 + tid, o);
+    if (tid == 0) part_store2(own_row, m, lsum);
+    __syncthreads();  // every store of the row has completed
+    if (tid == 0) {
+        const int done = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sm.state = (done == p1 - p0 - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (sm.state == 1 && w == 0) {
+        merge_rows(A.part, A.part_rows, p0, p1, h, H, A.out + (size_t(seq) * H + h) * D, l);
+        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
 // ---------------------------------------------------------------------------------------
-// shared_kernel: grid = n_items * H workgroups; an item = (segment of chunks, up to 16*MB
-// sequences).  The segment is one token stream cut into 16-token blocks; wave w takes blocks
-// w, w+4, ...  and keeps its own online-softmax state, so waves never wait for each other
-// until the final merge.
+// shared_path: an item = (segment of chunks, up to 32 sequences).  The segment is one token
+// stream cut into 16-token blocks; wave w takes blocks w, w+4, ... and keeps its own online-
+// softmax state, so waves never wait for each other until the final merge.  The next block's
+// K and V are requested before the current one is consumed.
 //
 // Matrix-core operand layout (v_mfma_f32_16x16x*: lane l = 16*g + i):
 //   A holds row i, B holds column i, each with the k-slice of group g; D holds rows 4g..4g+3
@@ -251,33 +432,25 @@ __global__ __launch_bounds__(WG) void stream_kernel(
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
 //   of the 16 x 128 V block read column-wise.
 // ---------------------------------------------------------------------------------------
-constexpr int VPITCH = D + 4;  // halves per LDS row of the V block: 264 B keeps the four
-                               // token groups on disjoint banks for 2-byte column reads
-constexpr int OPITCH = D + 4;  // floats per row of the cross-wave accumulation buffer
-
-template <int C, int MB>
-__global__ __launch_bounds__(WG) void shared_kernel(
-  const half_t* __restrict__ q, const half_t* __restrict__ kpool,
-  const half_t* __restrict__ vpool, float* __restrict__ part,
-  const WorkItem* __restrict__ items, const int32_t* __restrict__ slots,
-  const int32_t* __restrict__ seq_len, int delta_tokens, int H, float scale_log2) {
-    const int h = blockIdx.x % H;
-    const WorkItem it = items[blockIdx.x / H];
+template <int C>
+__device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem& it, int h,
+                                            SharedPathLds& sm) {
+    const half_t* __restrict__ kpool = A.kpool;
+    const half_t* __restrict__ vpool = A.vpool;
+    const int32_t* __restrict__ slots = A.slots;
+    const int H = A.H;
+    const float scale_log2 = A.scale_log2;
     const int tid = threadIdx.x;
     const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
-    const int len = seq_len[it.len_seq] + delta_tokens;
-
-    __shared__ __attribute__((aligned(16))) half_t sm_v[NW][16 * VPITCH];
-    __shared__ __attribute__((aligned(16))) float sm_o[MB * 16 * OPITCH];
-    __shared__ float sm_m[NW][MB * 16];
-    __shared__ float sm_l[NW][MB * 16];
+    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
+    const bool two = it.n_rows > 16;  // second 16-row block in use (uniform)
 
     // Q^T operand: sequence row mb*16+i, dims 32*ks + 8*g .. +7
     h8 qreg[MB][4];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
         const int row = mb * 16 + i;
-        const half_t* qp = q + (size_t(it.seq_begin + row) * H + h) * D + 8 * g;
+        const half_t* qp = A.q + (size_t(it.seq_begin + row) * H + h) * D + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
@@ -294,37 +467,51 @@ __global__ __launch_bounds__(WG) void shared_kernel(
         for (int db = 0; db < 8; db++) oacc[mb][db] = f4{ 0.f, 0.f, 0.f, 0.f };
     }
 
-    const int n_blocks = it.n_chunks * (C / 16);
-    for (int tb = w; tb < n_blocks; tb += NW) {
-        const int ck = tb / (C / 16);
-        const int row0 = (tb % (C / 16)) * 16;
-        int valid = len - (it.pos0 + ck) * C - row0;  // valid tokens in this block
-        if (valid <= 0) break;
-        const int slot = slots[it.slot_first + ck];
-        const size_t base = ((size_t(slot) * H + h) * size_t(C) + row0) * D;
-
-        h8 kreg[4];
+    constexpr int BPC = C / 16;  // blocks per chunk
+    const int n_blocks = it.n_chunks * BPC;
+    // valid tokens of block tb (<= 0: past the end of the sequence), and its element offset
+    auto block_valid = [&](int tb) { return len - (it.pos0 + tb / BPC) * C - (tb % BPC) * 16; };
+    auto block_base = [&](int tb) {
+        return ((size_t(slots[it.slot_first + tb / BPC]) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
+    };
+    h8 kreg[4], knext[4];
+    uint4 vraw[4], vnext[4];
+    auto load_block = [&](int tb, h8 (&kr)[4], uint4 (&vr)[4]) {
+        const size_t base = block_base(tb);
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            kreg[ks] = *reinterpret_cast<const h8*>(kpool + base + size_t(i) * D + 32 * ks + 8 * g);
+            kr[ks] = *reinterpret_cast<const h8*>(kpool + base + size_t(i) * D + 32 * ks + 8 * g);
         }
-        uint4 vraw[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) vr[r] = *(reinterpret_cast<const uint4*>(vpool + base) + 64 * r + l);
+    };
+
+    int tb = w;
+    bool have = tb < n_blocks && block_valid(tb) > 0;
+    if (have) load_block(tb, kreg, vraw);
+    while (have) {
+        const int valid = block_valid(tb);
+        const int tn = tb + NW;
+        const bool have_next = tn < n_blocks && block_valid(tn) > 0;
+        if (have_next) load_block(tn, knext, vnext);
+
+        // V block -> LDS rows (row 4r+g, dims 8i..8i+7); stale rows past the end are zeroed
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            vraw[r] = *(reinterpret_cast<const uint4*>(vpool + base) + 64 * r + l);
-            if (4 * r + g >= valid) vraw[r] = make_uint4(0, 0, 0, 0);  // stale rows past the end
-        }
-        // V block -> LDS rows (row 4r+g, dims 8i..8i+7)
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            uint2* dst = reinterpret_cast<uint2*>(&sm_v[w][(4 * r + g) * VPITCH + 8 * i]);
-            dst[0] = make_uint2(vraw[r].x, vraw[r].y);
-            dst[1] = make_uint2(vraw[r].z, vraw[r].w);
+            uint4 t = vraw[r];
+            if (4 * r + g >= valid) t = make_uint4(0, 0, 0, 0);
+            uint2* dst = reinterpret_cast<uint2*>(&sm.v[w][(4 * r + g) * VPITCH + 8 * i]);
+            dst[0] = make_uint2(t.x, t.y);
+            dst[1] = make_uint2(t.z, t.w);
         }
 
         h4 pb[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
+            if (mb == 1 && !two) {
+                pb[mb] = h4{ 0, 0, 0, 0 };
+                continue;
+            }
             f4 s = f4{ 0.f, 0.f, 0.f, 0.f };
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
@@ -358,14 +545,19 @@ __global__ __launch_bounds__(WG) void shared_kernel(
         // O^T += V^T . P^T : A = V^T (row = dim 16*db + i, k = tokens 4g..4g+3)
 #pragma unroll
         for (int db = 0; db < 8; db++) {
-            const half_t* col = &sm_v[w][(4 * g) * VPITCH + 16 * db + i];
+            const half_t* col = &sm.v[w][(4 * g) * VPITCH + 16 * db + i];
             const h4 a = h4{ col[0], col[VPITCH], col[2 * VPITCH], col[3 * VPITCH] };
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                oacc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[mb], oacc[mb][db], 0, 0, 0);
-            }
+            oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[0], oacc[0][db], 0, 0, 0);
+            if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1], oacc[1][db], 0, 0, 0);
         }
         __builtin_amdgcn_wave_barrier();
+
+        have = have_next;
+        tb = tn;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) kreg[ks] = knext[ks];
+#pragma unroll
+        for (int r = 0; r < 4; r++) vraw[r] = vnext[r];
     }
 
     // ---- merge the four waves ------------------------------------------------------------
@@ -373,18 +565,18 @@ __global__ __launch_bounds__(WG) void shared_kernel(
     for (int mb = 0; mb < MB; mb++) {
         l_lane[mb] += shfl_xor(l_lane[mb], 16);
         l_lane[mb] += shfl_xor(l_lane[mb], 32);
-        if (g == 0) sm_m[w][mb * 16 + i] = m_run[mb];
+        if (g == 0) sm.m[w][mb * 16 + i] = m_run[mb];
     }
     __syncthreads();
     float m_all[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
-        float m = sm_m[0][mb * 16 + i];
+        float m = sm.m[0][mb * 16 + i];
 #pragma unroll
-        for (int k = 1; k < NW; k++) m = fmaxf(m, sm_m[k][mb * 16 + i]);
+        for (int k = 1; k < NW; k++) m = fmaxf(m, sm.m[k][mb * 16 + i]);
         m_all[mb] = m;
         const float f = (m_run[mb] == NEG_INF) ? 0.f : fast_exp2(m_run[mb] - m);
-        if (g == 0) sm_l[w][mb * 16 + i] = l_lane[mb] * f;
+        if (g == 0) sm.l[w][mb * 16 + i] = l_lane[mb] * f;
 #pragma unroll
         for (int db = 0; db < 8; db++) oacc[mb][db] *= f;
     }
@@ -395,7 +587,7 @@ __global__ __launch_bounds__(WG) void shared_kernel(
 #pragma unroll
                 for (int db = 0; db < 8; db++) {
                     // lane owns dims 16*db + 4*g .. +3 of sequence row mb*16 + i
-                    f4* dst = reinterpret_cast<f4*>(&sm_o[(mb * 16 + i) * OPITCH + 16 * db + 4 * g]);
+                    f4* dst = reinterpret_cast<f4*>(&sm.o[(mb * 16 + i) * OPITCH + 16 * db + 4 * g]);
                     *dst = (k == 0) ? oacc[mb][db] : (*dst + oacc[mb][db]);
                 }
             }
@@ -406,8 +598,10 @@ __global__ __launch_bounds__(WG) void shared_kernel(
     // ---- write the partial rows ------------------------------------------------------------
     for (int idx = tid; idx < it.n_rows * (D / 4); idx += WG) {
         const int row = idx / (D / 4), c4 = idx % (D / 4);
-        float* dst = part + (size_t(it.part_row + row) * H + h) * PART_STRIDE;
-        *reinterpret_cast<f4*>(dst + 4 + 4 * c4) = *reinterpret_cast<const f4*>(&sm_o[row * OPITCH + 4 * c4]);
+        float* dst = A.part + (size_t(it.part_row + row) * H + h) * PART_STRIDE + 4 + 4 * c4;
+        const f4 v = *reinterpret_cast<const f4*>(&sm.o[row * OPITCH + 4 * c4]);
+        part_store2(dst, v[0], v[1]);
+        part_store2(dst + 2, v[2], v[3]);
     }
     if (w == 0 && g == 0) {
 #pragma unroll
@@ -416,18 +610,50 @@ __global__ __launch_bounds__(WG) void shared_kernel(
             if (row < it.n_rows) {
                 float lsum = 0.f;
 #pragma unroll
-                for (int k = 0; k < NW; k++) lsum += sm_l[k][row];
-                float* dst = part + (size_t(it.part_row + row) * H + h) * PART_STRIDE;
-                dst[0] = m_all[mb];
-                dst[1] = lsum;
+                for (int k = 0; k < NW; k++) lsum += sm.l[k][row];
+                part_store2(A.part + (size_t(it.part_row + row) * H + h) * PART_STRIDE, m_all[mb], lsum);
             }
+        }
+    }
+    if (!A.fuse_merge) return;
+
+    // count one finished partial for every covered sequence (after the barrier: all stores of
+    // the rows have completed); merge the completed ones
+    __syncthreads();
+    if (tid < it.n_rows) {
+        const int s = it.seq_begin + tid;
+        const int done = __hip_atomic_fetch_add(&A.counters[s * H + h], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sm.last[tid] = (done == A.part_ptr[s + 1] - A.part_ptr[s] - 1);
+    }
+    __syncthreads();
+    for (int r = w; r < it.n_rows; r += NW) {
+        if (sm.last[r]) {
+            const int s = it.seq_begin + r;
+            merge_rows(A.part, A.part_rows, A.part_ptr[s], A.part_ptr[s + 1], h, H,
+                       A.out + (size_t(s) * H + h) * D, l);
+            if (l == 0) __hip_atomic_store(&A.counters[s * H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
 
-// ---------------------------------------------------------------------------------------
-// merge_kernel: one wave per (sequence, head); lane owns two output dims.
-// ---------------------------------------------------------------------------------------
+// grid = (n_shared_items + n_stream_items) * H workgroups, shared items first: they have the
+// longest dependent chains and are sized to about one per compute unit, so they are done long
+// before the streaming is and the merge falls to stream workgroups, one row each.
+template <int C>
+__global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
+    __shared__ DecodeLds lds;
+    const int bid = blockIdx.x;
+    if (bid < A.n_shared_wgs) {
+        const WorkItem it = A.shared_items[bid / A.H];
+        shared_path<C>(A, it, bid % A.H, lds.sh);
+    } else {
+        const int sid = bid - A.n_shared_wgs;
+        const WorkItem it = A.stream_items[sid / A.H];
+        stream_path<C>(A, it, sid % A.H, lds.st);
+    }
+}
+
+// one wave per (sequence, head)
 __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ part,
                                                    half_t* __restrict__ out,
                                                    const int32_t* __restrict__ part_ptr,
@@ -439,25 +665,12 @@ __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ par
     const int seq = sh / H, h = sh % H;
     const int p0 = part_ptr[seq], p1 = part_ptr[seq + 1];
     if (p0 == p1) return;  // written directly by a stream item
+    merge_rows(part, part_rows, p0, p1, h, H, out + (size_t(seq) * H + h) * D, l);
+}
 
-    float m = NEG_INF;
-    for (int p = p0 + l; p < p1; p += 64) {
-        m = fmaxf(m, part[(size_t(part_rows[p]) * H + h) * PART_STRIDE]);
-    }
-    m = wave_max(m);
-    float lsum = 0.f;
-    f2 o = f2{ 0.f, 0.f };
-    for (int p = p0; p < p1; p++) {
-        const float* row = part + (size_t(part_rows[p]) * H + h) * PART_STRIDE;
-        const float mp = row[0];
-        const float f = (mp == NEG_INF) ? 0.f : fast_exp2(mp - m);
-        lsum += f * row[1];
-        const f2 v = *reinterpret_cast<const f2*>(row + 4 + 2 * l);
-        o += f * v;
-    }
-    const float r = lsum > 0.f ? 1.f / lsum : 0.f;
-    h2* dst = reinterpret_cast<h2*>(out + (size_t(seq) * H + h) * D + 2 * l);
-    *dst = h2{ half_t(o[0] * r), half_t(o[1] * r) };
+__global__ __launch_bounds__(WG) void fill_kernel(int32_t* __restrict__ p, int n, int32_t value) {
+    const int idx = blockIdx.x * WG + threadIdx.x;
+    if (idx < n) p[idx] = value;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -512,77 +725,58 @@ __global__ __launch_bounds__(WG) void scatter_kernel(const T* __restrict__ k, co
         if (e_ != hipSuccess) return static_cast<int>(e_);       \
     } while (0)
 
-int launch_stream(const LaunchArgs& a, const WorkItem* items, int n_items, hipStream_t st) {
-    if (n_items <= 0) return 0;
-    const dim3 grid(static_cast<unsigned>(n_items) * a.H), block(WG);
-    const half_t* q = static_cast<const half_t*>(a.q);
-    const half_t* kp = static_cast<const half_t*>(a.kpool);
-    const half_t* vp = static_cast<const half_t*>(a.vpool);
-    half_t* out = static_cast<half_t*>(a.out);
-    switch (a.C) {
-        case 32:
-            hipLaunchKernelGGL(stream_kernel<32>, grid, block, 0, st, q, kp, vp, out, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        case 64:
-            hipLaunchKernelGGL(stream_kernel<64>, grid, block, 0, st, q, kp, vp, out, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        case 128:
-            hipLaunchKernelGGL(stream_kernel<128>, grid, block, 0, st, q, kp, vp, out, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        default:
-            return -1;
-    }
-    CA_LAUNCH_CHECK();
-    return 0;
+static DecodeArgs decode_args(const LaunchArgs& a) {
+    DecodeArgs d;
+    d.q = static_cast<const half_t*>(a.q);
+    d.kpool = static_cast<const half_t*>(a.kpool);
+    d.vpool = static_cast<const half_t*>(a.vpool);
+    d.out = static_cast<half_t*>(a.out);
+    d.part = a.part;
+    d.shared_items = a.shared_items;
+    d.stream_items = a.stream_items;
+    d.slots = a.slots;
+    d.seq_len = a.seq_len;
+    d.part_ptr = a.part_ptr;
+    d.part_rows = a.part_rows;
+    d.counters = a.counters;
+    d.n_shared_wgs = 0;
+    d.delta_tokens = a.delta_tokens;
+    d.H = a.H;
+    d.scale_log2 = a.scale_log2;
+    d.fuse_merge = 0;
+    return d;
 }
 
-template <int C>
-static int launch_shared_c(const LaunchArgs& a, const WorkItem* items, int n_items, int mb,
-                           hipStream_t st) {
-    const dim3 grid(static_cast<unsigned>(n_items) * a.H), block(WG);
-    const half_t* q = static_cast<const half_t*>(a.q);
-    const half_t* kp = static_cast<const half_t*>(a.kpool);
-    const half_t* vp = static_cast<const half_t*>(a.vpool);
-    switch (mb) {
-        case 1:
-            hipLaunchKernelGGL((shared_kernel<C, 1>), grid, block, 0, st, q, kp, vp, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        case 2:
-            hipLaunchKernelGGL((shared_kernel<C, 2>), grid, block, 0, st, q, kp, vp, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        case 4:
-            hipLaunchKernelGGL((shared_kernel<C, 4>), grid, block, 0, st, q, kp, vp, a.part, items,
-                               a.slots, a.seq_len, a.delta_tokens, a.H, a.scale_log2);
-            break;
-        default:
-            return -1;
-    }
-    CA_LAUNCH_CHECK();
-    return 0;
-}
-
-int launch_shared(const LaunchArgs& a, const WorkItem* items, int n_items, int mb,
+int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, bool fuse_merge,
                   hipStream_t st) {
-    if (n_items <= 0) return 0;
+    const int64_t wgs = int64_t(n_shared_items + n_stream_items) * a.H;
+    if (wgs <= 0) return 0;
+    DecodeArgs d = decode_args(a);
+    d.n_shared_wgs = n_shared_items * a.H;
+    d.fuse_merge = fuse_merge ? 1 : 0;
+    const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
     switch (a.C) {
-        case 32: return launch_shared_c<32>(a, items, n_items, mb, st);
-        case 64: return launch_shared_c<64>(a, items, n_items, mb, st);
-        case 128: return launch_shared_c<128>(a, items, n_items, mb, st);
+        case 32: hipLaunchKernelGGL(decode_kernel<32>, grid, block, 0, st, d); break;
+        case 64: hipLaunchKernelGGL(decode_kernel<64>, grid, block, 0, st, d); break;
+        case 128: hipLaunchKernelGGL(decode_kernel<128>, grid, block, 0, st, d); break;
         default: return -1;
     }
+    CA_LAUNCH_CHECK();
+    return 0;
 }
 
-int launch_merge(const LaunchArgs& a, const int32_t* part_ptr, const int32_t* part_rows,
-                 int n_seqs, hipStream_t st) {
+int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st) {
     if (n_seqs <= 0) return 0;
     const int waves = n_seqs * a.H;
     hipLaunchKernelGGL(merge_kernel, dim3((waves + NW - 1) / NW), dim3(WG), 0, st, a.part,
-                       static_cast<half_t*>(a.out), part_ptr, part_rows, n_seqs, a.H);
+                       static_cast<half_t*>(a.out), a.part_ptr, a.part_rows, n_seqs, a.H);
+    CA_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(fill_kernel, dim3((n + WG - 1) / WG), dim3(WG), 0, st, p, n, value);
     CA_LAUNCH_CHECK();
     return 0;
 }

@@ -107,9 +107,10 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     }
     int seg_chunks = params.shared_seg_chunks;
     if (seg_chunks <= 0) {
-        // aim at about two workgroups per compute unit, but keep segments between 1 and 16
-        // chunks: longer segments mean fewer partial rows to write and merge
-        const int64_t target = int64_t(2) * params.n_cus;
+        // aim at about one workgroup per compute unit, but keep segments between 1 and 16
+        // chunks: the shared workgroups then leave room for streaming ones from the start, and
+        // longer segments mean fewer partial rows to write and merge
+        const int64_t target = params.n_cus;
         const int64_t wgs_at_1 = shared_units * std::max(params.n_heads, 1);
         seg_chunks = static_cast<int>(std::clamp<int64_t>(wgs_at_1 / std::max<int64_t>(target, 1), 1, 16));
     }
@@ -161,7 +162,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         // shrink towards four when there would be too few workgroups to fill the device
         const int per_wg_tokens = 512;
         stream_chunks = std::max(4, per_wg_tokens / chunk_size);
-        const int64_t target = int64_t(4) * params.n_cus;
+        const int64_t target = int64_t(2) * params.n_cus;
         while (stream_chunks > 4 &&
                (stream_chunk_total / stream_chunks) * std::max(params.n_heads, 1) < target) {
             stream_chunks /= 2;
@@ -177,7 +178,9 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             }
         }
         const int total = static_cast<int>(own.size());
-        const int n_items = ceil_div(total, stream_chunks);
+        // the last chunk is the sequence's tail, usually far from full: it rides along with
+        // the item before it instead of opening a new one
+        const int n_items = std::max(1, ceil_div(total - 1, stream_chunks));
         for (int g = 0; g < n_items; g++) {
             const int c0 = int(int64_t(total) * g / n_items);
             const int c1 = int(int64_t(total) * (g + 1) / n_items);

@@ -59,7 +59,7 @@ struct PlanParams {
     int n_cus = 256;
 };
 
-constexpr int kMaxRows = 64;  // sequences per shared work item (M tile)
+constexpr int kMaxRows = 32;  // sequences per shared work item (M tile)
 
 struct Plan {
     int n_seqs = 0;

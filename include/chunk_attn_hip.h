@@ -108,12 +108,13 @@ int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
  * reference's partial buffers. */
 int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
 
-/* Per-phase timing of ca_attention, measured with HIP events recorded on the stream the
- * kernels are launched on (the reference marks the same phases with NVTX ranges,
- * kernel_cuda.cu:1334-1433).  While enabled, every ca_attention call records four events;
- * ca_ctx_read_timing waits for the last call and returns the accumulated milliseconds of the
- * chunk-first launches, the sequence-first launch and the merge launch. */
-int ca_ctx_set_timing(ca_ctx* ctx, int enable);
+/* Timing of ca_attention with HIP events recorded on the stream the kernels are launched on
+ * (the reference marks its phases with NVTX ranges, kernel_cuda.cu:1334-1433).
+ * mode 0: off.  mode 1: every ca_attention call is bracketed by two events; ca_ctx_read_timing
+ * returns the accumulated milliseconds of the fused launch in *shared_ms (the other two stay 0).
+ * mode 2: ca_attention runs as three separately timed launches (chunk-first, sequence-first,
+ * merge) and the three accumulators are filled; for phase analysis, slower than the fused launch. */
+int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
 
@@ -145,6 +146,10 @@ int ca_ctx_ref_tables(const ca_ctx* ctx, int32_t* final_idx, int32_t* slots, int
  * natural-log units of score/sqrt(d).  Needs tables built with shared_seg_chunks = 1 and
  * partition 0.  Synchronises the stream. */
 int ca_ctx_export_partials(ca_ctx* ctx, float* maxs, float* sums, float* attns, void* stream);
+
+/* Raw copy of the partial-row buffer ([n_part_rows][n_heads][160] floats: max, sum, 2 unused,
+ * 128 acc in base-2 units, 28 unused) to the host, for inspection.  Synchronises the stream. */
+int ca_ctx_read_partials_raw(ca_ctx* ctx, float* out, int64_t n_floats, void* stream);
 
 /* ---- host-only table builder (no device needed) ---------------------------------------- */
 
