@@ -55,6 +55,13 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // whose L2 is not coherent with the writer's.  They are therefore moved with device-scope
 // relaxed atomics (write-through stores, L2-bypassing loads): no cache-wide fence is needed,
 // only "stores done" (a workgroup barrier) before the completion counter is bumped.
+// Before a workgroup announces its partial rows through the completion counter, every wave
+// waits until its own stores have been acknowledged: a workgroup barrier alone orders waves
+// but does not wait for their outstanding global stores.
+__device__ __forceinline__ void wait_own_stores() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0)
+}
 __device__ __forceinline__ void part_store(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -208,9 +215,7 @@ struct StreamPathLds {
     float o[NW][D];
     float m[NW];
     float l[NW];
-    float own_o[D];  // the workgroup's combined result, kept for the in-place merge
-    float own_m, own_l;
-    int state;       // 0: not last, 1: last after publishing the partial, 2: last without publishing
+    int state;  // workgroup-uniform decision flags
 };
 union __attribute__((aligned(16))) DecodeLds {
     SharedPathLds sh;
@@ -241,6 +246,59 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = 0.f;
+
+    // Folding in the other partial rows of this (sequence, head).  Once every other partial
+    // is complete (the counter says so and stays so until this workgroup resets it), wave w
+    // folds rows w, w+4, ... of the list straight into its running softmax state, so nothing
+    // is published and nothing remains to merge.  Each wave tries once after its first tile,
+    // when the row loads hide behind the streaming; the rest happens at the end.
+    const bool can_fold = A.fuse_merge && it.part_row >= 0;
+    const int p0 = can_fold ? A.part_ptr[seq] : 0;
+    const int p1 = can_fold ? A.part_ptr[seq + 1] : 0;
+    int* counter = A.counters + (seq * H + h);
+    bool folded = !can_fold;
+    auto fold_rows = [&]() {
+        for (int pb = p0 + w; pb < p1; pb += 2 * NW) {
+            // two rows per round so that their loads overlap
+            float rm[2], rl[2];
+            f2 rv[2][4];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int p = pb + u * NW;
+                rm[u] = NEG_INF;
+                rl[u] = 0.f;
+                const int row = (p < p1) ? A.part_rows[p] : it.part_row;
+                if (row != it.part_row) {
+                    const float* r = A.part + (size_t(row) * H + h) * PART_STRIDE;
+                    const f2 ml = part_load2(r);
+                    rm[u] = ml[0];
+                    rl[u] = ml[1];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rv[u][e] = part_load2(r + 4 + 8 * j + 2 * e);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rv[u][e] = f2{ 0.f, 0.f };
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                if (rm[u] == NEG_INF) continue;  // empty or absent row (wave-uniform)
+                const float mn = fmaxf(m_run, rm[u]);
+                const float fa = (m_run == NEG_INF) ? 0.f : fast_exp2(m_run - mn);
+                const float fb = fast_exp2(rm[u] - mn);
+                const float fo = (g == 0) ? fb : 0.f;  // the row is added once, by lane group 0
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    acc[2 * e] = acc[2 * e] * fa + fo * rv[u][e][0];
+                    acc[2 * e + 1] = acc[2 * e + 1] * fa + fo * rv[u][e][1];
+                }
+                l_lane = l_lane * fa + ((l == 0) ? fb * rl[u] : 0.f);
+                m_run = mn;
+            }
+        }
+        folded = true;
+    };
+    bool tried = !can_fold;
 
     for (int t = w; t < it.n_chunks; t += NW) {
         int valid = len - (it.pos0 + t) * C;
@@ -302,7 +360,26 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
                 for (int e = 0; e < 8; e++) acc[e] = __builtin_fmaf(pr[i], float(vv[e]), acc[e]);
             }
         }
+        if (!tried) {
+            tried = true;
+            const int done = __builtin_amdgcn_readfirstlane(
+              __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            if (done == p1 - p0 - 1) fold_rows();
+        }
     }
+
+    // end of streaming: one workgroup-uniform look at the counter decides between folding the
+    // remaining rows now and publishing this workgroup's partial.  The barrier in front makes
+    // the look later than every wave's own early look, so "complete" seen there is seen here.
+    if (can_fold) {
+        __syncthreads();
+        if (tid == 0) {
+            sm.state = (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p1 - p0 - 1);
+        }
+        __syncthreads();
+        if (sm.state && !folded) fold_rows();
+    }
+    const bool complete = can_fold && sm.state;
 
     // wave result: rows are spread over the four 16-lane groups
     const float l_wave = wave_sum(l_lane);
@@ -334,86 +411,28 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
             lsum += f * sm.l[k];
         }
     }
-    if (it.part_row < 0) {  // nothing else to merge: final output
+    if (it.part_row < 0 || complete) {  // nothing (left) to merge: final output
         if (tid < D) {
             const float r = lsum > 0.f ? 1.f / lsum : 0.f;
             A.out[(size_t(seq) * H + h) * D + tid] = half_t(o * r);
         }
+        if (complete && tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
     float* own_row = A.part + (size_t(it.part_row) * H + h) * PART_STRIDE;
-    if (!A.fuse_merge) {
-        if (tid < D) part_store(own_row + 4 + tid, o);
-        if (tid == 0) part_store2(own_row, m, lsum);
-        return;
-    }
-
-    // Fused merge.  If every other partial of this (sequence, head) is already complete, merge
-    // straight from LDS without publishing this one; otherwise publish, count, and let whoever
-    // arrives last merge from memory.
-    const int p0 = A.part_ptr[seq], p1 = A.part_ptr[seq + 1];
-    int* counter = &A.counters[seq * H + h];
-    if (tid == 0) {
-        sm.state = (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p1 - p0 - 1) ? 2 : 0;
-    }
-    if (tid < D) sm.own_o[tid] = o;
-    if (tid == 0) {
-        sm.own_m = m;
-        sm.own_l = lsum;
-    }
-    __syncthreads();
-    if (sm.state == 2) {
-        // wave w folds partial rows w, w+4, ... (not our own) into a running (m, l, acc)
-        float mw = NEG_INF, lw = 0.f;
-        f2 ow = f2{ 0.f, 0.f };
-        for (int p = p0 + w; p < p1; p += NW) {
-            const int row = A.part_rows[p];
-            if (row == it.part_row) continue;
-            const float* r = A.part + (size_t(row) * H + h) * PART_STRIDE;
-            const f2 ml = part_load2(r);
-            const f2 v = part_load2(r + 4 + 2 * l);
-            const float mn = fmaxf(mw, ml[0]);
-            const float fa = (mw == NEG_INF) ? 0.f : fast_exp2(mw - mn);
-            const float fb = (ml[0] == NEG_INF) ? 0.f : fast_exp2(ml[0] - mn);
-            ow = fa * ow + fb * v;
-            lw = fa * lw + fb * ml[1];
-            mw = mn;
-        }
-        __syncthreads();  // everyone has read sm.o / sm.m / sm.l of the first combine
-        sm.o[w][2 * l] = ow[0];
-        sm.o[w][2 * l + 1] = ow[1];
-        if (l == 0) {
-            sm.m[w] = mw;
-            sm.l[w] = lw;
-        }
-        __syncthreads();
-        if (tid < D) {
-            float mm = sm.own_m;
-#pragma unroll
-            for (int k = 0; k < NW; k++) mm = fmaxf(mm, sm.m[k]);
-            const float f0 = (sm.own_m == NEG_INF) ? 0.f : fast_exp2(sm.own_m - mm);
-            float oo = f0 * sm.own_o[tid], ll = f0 * sm.own_l;
-#pragma unroll
-            for (int k = 0; k < NW; k++) {
-                const float f = (sm.m[k] == NEG_INF) ? 0.f : fast_exp2(sm.m[k] - mm);
-                oo += f * sm.o[k][tid];
-                ll += f * sm.l[k];
-            }
-            const float r = ll > 0.f ? 1.f / ll : 0.f;
-            A.out[(size_t(seq) * H + h) * D + tid] = half_t(oo * r);
-        }
-        if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return;
-    }
     if (tid < D) part_store(own_row + 4 + tid, o);
     if (tid == 0) part_store2(own_row, m, lsum);
+    if (!A.fuse_merge) return;
+
+    // publish, count, and let whoever arrives last merge from memory
+    wait_own_stores();
     __syncthreads();  // every store of the row has completed
     if (tid == 0) {
         const int done = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        sm.state = (done == p1 - p0 - 1) ? 1 : 0;
+        sm.state = (done == p1 - p0 - 1);
     }
     __syncthreads();
-    if (sm.state == 1 && w == 0) {
+    if (sm.state && w == 0) {
         merge_rows(A.part, A.part_rows, p0, p1, h, H, A.out + (size_t(seq) * H + h) * D, l);
         if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -619,6 +638,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
 
     // count one finished partial for every covered sequence (after the barrier: all stores of
     // the rows have completed); merge the completed ones
+    wait_own_stores();
     __syncthreads();
     if (tid < it.n_rows) {
         const int s = it.seq_begin + tid;
