@@ -68,6 +68,21 @@ def phase_times(attn, q, out, steps, torch, mode, partition=0):
     return {k: t[k] / n for k in ("shared_ms", "stream_ms", "merge_ms")}
 
 
+def measured_traffic(workload, info):
+    """HBM bytes per decode launch from the committed rocprofv3 --pmc summary, when it was taken
+    for this workload with this work list; None otherwise (counters cannot be read from here)."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter summary"
+    e = table.get(workload)
+    if not e or e.get("shared_items") != info.n_shared_items or e.get("stream_items") != info.n_stream_items:
+        return None, "no counter summary for this workload / work list"
+    return int(e["decode_kernel_bytes"]), e.get("how", "")
+
+
 def cpu_baseline(attn, q_np, budget_s, torch):
     """The CPU restatement of the reference's MKL path on the same cache contents (fp16 values
     widened to fp32), timed on this machine's host cores."""
@@ -106,7 +121,10 @@ def main() -> int:
     ap.add_argument("--no-paged", action="store_true", help="skip the private-copies baseline")
     ap.add_argument("--seg-chunks", type=int, default=0)
     ap.add_argument("--stream-chunks", type=int, default=0)
+    ap.add_argument("--schedule", type=int, default=0, help="0 producer launch + merge launch (default), 1 single launch with in-kernel merge")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="only run 20 plain device copies of this many MiB (a known-size reference for HBM traffic counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the decode path has no multi-GPU component (run with --gpus 1)", file=sys.stderr)
@@ -120,16 +138,29 @@ def main() -> int:
         return 3
     torch.cuda.set_device(0)
 
+    if args.calibrate_copy > 0:
+        n = args.calibrate_copy << 20
+        src = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_MiB": args.calibrate_copy, "copies": 20, "bytes_read_per_copy": n, "bytes_written_per_copy": n}))
+        return 0
+
     w = synth.baseline_config(args.config, args.fraction)
     attn = build_cache(w, torch, capi, args.seed)
     if args.seg_chunks or args.stream_chunks:
         attn.ctx.set_plan(args.seg_chunks, args.stream_chunks)
+    attn.ctx.set_schedule(args.schedule)
     q_np = w.q(args.seed)
     q = torch.from_numpy(q_np).to("cuda:0")
     out = torch.empty_like(q)
 
     ms = time_forward(attn, q, out, args.steps, args.warmup, torch)
-    fused_ms = phase_times(attn, q, out, min(args.steps, 100), torch, 1)["shared_ms"]
+    normal = phase_times(attn, q, out, min(args.steps, 100), torch, 1)
+    decode_ms, merge_ms = normal["shared_ms"], normal["merge_ms"]
     ph = phase_times(attn, q, out, min(args.steps, 50), torch, 2)
     info = attn.ctx.plan_info()
     H, d = w.n_heads, w.d_head
@@ -138,8 +169,10 @@ def main() -> int:
     shared_bytes = tok_bytes * info.shared_tokens
     qo_bytes = 4 * w.n_seqs * H * d
     step_bytes = stream_bytes + shared_bytes + qo_bytes
-    # the forward is one launch: its algorithmic bytes are every attended K/V row once plus Q and O
-    achieved = step_bytes / (fused_ms * 1e-3) / 1e9 if fused_ms > 0 else 0.0
+    # dominant kernel = the decode launch: it reads every attended K/V row once, plus Q
+    decode_bytes = stream_bytes + shared_bytes + qo_bytes // 2
+    achieved = decode_bytes / (decode_ms * 1e-3) / 1e9 if decode_ms > 0 else 0.0
+    traffic, traffic_note = measured_traffic(w.name, info)
     stream_gbps = stream_bytes / (ph["stream_ms"] * 1e-3) / 1e9 if ph["stream_ms"] > 0 else 0.0
 
     result = {
@@ -165,9 +198,11 @@ def main() -> int:
         "split_phases_us": {k.replace("_ms", ""): round(v * 1e3, 2) for k, v in ph.items()},
         "unique_kv_streaming": {"GBps": round(stream_gbps, 1), "frac_of_hbm_peak": round(stream_gbps / HBM_PEAK_GBPS, 4),
                                 "bytes": stream_bytes, "note": "sequence-first phase launched alone, HIP events"},
+        "launches_us": {"decode_kernel": round(decode_ms * 1e3, 2), "merge_kernel": round(merge_ms * 1e3, 2)},
         "roofline": {"bound": "hbm", "kernel": "decode_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "bytes_per_launch": step_bytes, "avg_launch_us": round(fused_ms * 1e3, 2)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "traffic_note": traffic_note,
+                     "bytes_per_launch": decode_bytes, "avg_launch_us": round(decode_ms * 1e3, 2)},
     }
 
     if not args.no_paged:

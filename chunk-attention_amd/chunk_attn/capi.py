@@ -63,6 +63,7 @@ SIGNATURES = {
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
+    "ca_ctx_set_schedule": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_read_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
@@ -76,9 +77,9 @@ SIGNATURES = {
                         [ctypes.c_int] * 9),
     "ca_tables_destroy": (None, [ctypes.c_void_p]),
     "ca_tables_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
-    "ca_tables_plan_sizes": (ctypes.c_int, [ctypes.c_void_p, c_int_p, c_int_p]),
+    "ca_tables_plan_sizes": (ctypes.c_int, [ctypes.c_void_p, c_int_p]),
     "ca_tables_ref": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
-    "ca_tables_plan": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 8),
+    "ca_tables_plan": (ctypes.c_int, [ctypes.c_void_p] + [c_i32_p] * 7),
     "ca_tree_create": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int,
                                       ctypes.c_int]),
     "ca_tree_destroy": (None, [ctypes.c_void_p]),
@@ -241,7 +242,7 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
                  n_heads: int = 32, n_cus: int = 256) -> dict:
     """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
     (work items as [n, 8] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
-    len_seq, reserved)."""
+    len_seq, reserved; an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
     lib = load()
     rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
     h = ctypes.c_void_p()
@@ -251,8 +252,8 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
     try:
         info = PlanInfo()
         _check(lib.ca_tables_info(h, ctypes.byref(info)))
-        n_slots, n_list = ctypes.c_int(), ctypes.c_int()
-        _check(lib.ca_tables_plan_sizes(h, ctypes.byref(n_slots), ctypes.byref(n_list)))
+        n_slots = ctypes.c_int()
+        _check(lib.ca_tables_plan_sizes(h, ctypes.byref(n_slots)))
         t = {
             "final_idx": np.zeros(info.n_chunks, np.int32),
             "slots": np.zeros(info.n_chunks, np.int32),
@@ -273,13 +274,11 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
             "slots": np.zeros(n_slots.value, np.int32),
             "seq_len": np.zeros(info.n_seqs, np.int32),
             "part_ptr": np.zeros(info.n_seqs + 1, np.int32),
-            "part_rows": np.zeros(n_list.value, np.int32),
             "tail_slot": np.zeros(info.n_seqs, np.int32),
             "tail_fill": np.zeros(info.n_seqs, np.int32),
         }
         _check(lib.ca_tables_plan(h, *[p[k].ctypes.data_as(c_i32_p) for k in (
-            "shared_items", "stream_items", "slots", "seq_len", "part_ptr", "part_rows",
-            "tail_slot", "tail_fill")]))
+            "shared_items", "stream_items", "slots", "seq_len", "part_ptr", "tail_slot", "tail_fill")]))
         p["n_part_rows"] = info.n_part_rows
         p["shared_tokens"] = info.shared_tokens
         p["stream_tokens"] = info.stream_tokens
@@ -346,6 +345,10 @@ class KernelContext:
 
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
+
+    def set_schedule(self, mode: int) -> None:
+        """0: producer launch + merge launch (default); 1: single launch, last finisher merges."""
+        _check(self._lib.ca_ctx_set_schedule(self._h, int(mode)))
 
     def set_timing(self, mode: int) -> None:
         """0 off, 1 time the fused launch, 2 run and time the three phases separately."""

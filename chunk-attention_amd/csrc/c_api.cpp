@@ -90,7 +90,8 @@ struct ca_ctx {
     int next_host = 0;
     // offsets into dev_blob
     size_t off_shared = 0, off_stream = 0, off_slots = 0, off_seq_len = 0, off_part_ptr = 0,
-           off_part_rows = 0, off_tail_slot = 0, off_tail_fill = 0;
+           off_tail_slot = 0, off_tail_fill = 0;
+    int schedule = 0;  // 0: partial-producing launch + merge launch; 1: one launch, last finisher merges
 
     float* part = nullptr;
     size_t part_cap = 0;  // bytes
@@ -131,7 +132,6 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.slots = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_slots);
     a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
     a.part_ptr = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr);
-    a.part_rows = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_rows);
     a.counters = c->counters;
     a.delta_tokens = c->delta_tokens;
     a.H = c->H;
@@ -170,7 +170,6 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     c->off_slots = place(p.slots.size() * 4);
     c->off_seq_len = place(p.seq_len.size() * 4);
     c->off_part_ptr = place(p.part_ptr.size() * 4);
-    c->off_part_rows = place(p.part_rows.size() * 4);
     c->off_tail_slot = place(p.tail_slot.size() * 4);
     c->off_tail_fill = place(p.tail_fill.size() * 4);
     const size_t total = std::max<size_t>(off, 64);
@@ -197,7 +196,6 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     put(c->off_slots, p.slots.data(), p.slots.size() * 4);
     put(c->off_seq_len, p.seq_len.data(), p.seq_len.size() * 4);
     put(c->off_part_ptr, p.part_ptr.data(), p.part_ptr.size() * 4);
-    put(c->off_part_rows, p.part_rows.data(), p.part_rows.size() * 4);
     put(c->off_tail_slot, p.tail_slot.data(), p.tail_slot.size() * 4);
     put(c->off_tail_fill, p.tail_fill.data(), p.tail_fill.size() * 4);
     CA_HIP(hipMemcpyAsync(c->dev_blob, hbuf, total, hipMemcpyHostToDevice, st));
@@ -261,13 +259,19 @@ int run_stream(ca_ctx* c, const void* q, void* out, hipStream_t st) {
 }
 
 int run_merge(ca_ctx* c, void* out, hipStream_t st) {
-    if (c->plan.part_rows.empty()) return CA_OK;
+    if (c->plan.n_part_rows == 0) return CA_OK;
     const ca::LaunchArgs a = launch_args(c, nullptr, out);
     return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
 }
 
 int run_fused(ca_ctx* c, const void* q, void* out, hipStream_t st) {
     const ca::LaunchArgs a = launch_args(c, q, out);
+    if (c->schedule == 0) {
+        // both phases in one launch (shared and stream workgroups overlap), then the merge
+        if (int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                                 static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch")) return rc;
+        return run_merge(c, out, st);
+    }
     return launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
                                        static_cast<int>(c->plan.stream_items.size()), true, st),
                      "decode launch");
@@ -381,7 +385,15 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
         if (!c->timing) return run_fused(c, q, out, st);
         if (int rc = collect_timing(c)) return rc;
         CA_HIP(hipEventRecord(c->ev[0], st));
-        if (c->timing == 1) {
+        if (c->timing == 1 && c->schedule == 0) {
+            // the forward as it normally runs: decode launch, then merge launch
+            const ca::LaunchArgs a = launch_args(c, q, out);
+            if (int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                                     static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch")) return rc;
+            CA_HIP(hipEventRecord(c->ev[1], st));
+            CA_HIP(hipEventRecord(c->ev[2], st));
+            if (int rc = run_merge(c, out, st)) return rc;
+        } else if (c->timing == 1) {
             if (int rc = run_fused(c, q, out, st)) return rc;
             CA_HIP(hipEventRecord(c->ev[1], st));
             CA_HIP(hipEventRecord(c->ev[2], st));
@@ -489,6 +501,12 @@ int ca_ctx_set_plan(ca_ctx* c, int shared_seg_chunks, int stream_chunks) {
     return CA_OK;
 }
 
+int ca_ctx_set_schedule(ca_ctx* c, int mode) {
+    if (!c || mode < 0 || mode > 1) return fail(CA_ERR_INVALID, "schedule mode must be 0 or 1");
+    c->schedule = mode;
+    return CA_OK;
+}
+
 int ca_ctx_plan_info(const ca_ctx* c, ca_plan_info* info) {
     if (!c || !info) return fail(CA_ERR_INVALID, "bad argument");
     info->n_seqs = c->n_seqs;
@@ -539,15 +557,24 @@ int ca_ctx_export_partials(ca_ctx* c, float* maxs, float* sums, float* attns, vo
         if (bytes) CA_HIP(hipMemcpyAsync(host.data(), c->part, bytes, hipMemcpyDeviceToHost, st));
         CA_HIP(hipStreamSynchronize(st));
         const float ln2 = 0.6931471805599453f;
-        // With one chunk per segment, segment k is the k-th shared chunk and its partial rows
-        // start at the reference's offsets[k]: both count n per shared chunk in row order.
-        for (int k = 0; k < c->ref.n_shared; k++) {
-            const int off = c->ref.offsets[k];
-            const int n = c->ref.ends[k] - c->ref.begins[k];
+        // With one chunk per segment the shared items come in shared-chunk order (several
+        // items per chunk when it covers more than one tile of sequences).  Sequence s keeps
+        // the partial of an item at row part_ptr[s] + item.part_row.
+        int chunk = -1, prev_slot_first = -1;
+        for (const auto& it : p.shared_items) {
+            if (it.slot_first != prev_slot_first) {
+                chunk++;
+                prev_slot_first = it.slot_first;
+            }
+            if (chunk >= c->ref.n_shared) return fail(CA_ERR_STATE, "shared items do not match the shared chunks");
+            const int off = c->ref.offsets[chunk];
+            const int b = c->ref.begins[chunk];
+            const int n = c->ref.ends[chunk] - b;
             for (int h = 0; h < c->H; h++) {
-                for (int r = 0; r < n; r++) {
-                    const float* src = host.data() + (size_t(off + r) * c->H + h) * ca::PART_STRIDE;
-                    const size_t dst = size_t(off) * c->H + size_t(h) * n + r;
+                for (int r = 0; r < it.n_rows; r++) {
+                    const int s = it.seq_begin + r;
+                    const float* src = host.data() + (size_t(p.part_ptr[s] + it.part_row) * c->H + h) * ca::PART_STRIDE;
+                    const size_t dst = size_t(off) * c->H + size_t(h) * n + (s - b);
                     if (maxs) maxs[dst] = src[0] * ln2;
                     if (sums) sums[dst] = src[1];
                     if (attns) std::memcpy(attns + dst * c->d, src + 4, sizeof(float) * c->d);
@@ -623,10 +650,9 @@ int ca_tables_info(const ca_tables* t, ca_plan_info* info) {
     return CA_OK;
 }
 
-int ca_tables_plan_sizes(const ca_tables* t, int* n_slots, int* n_part_list) {
+int ca_tables_plan_sizes(const ca_tables* t, int* n_slots) {
     if (!t) return fail(CA_ERR_INVALID, "bad argument");
     if (n_slots) *n_slots = static_cast<int>(t->plan.slots.size());
-    if (n_part_list) *n_part_list = static_cast<int>(t->plan.part_rows.size());
     return CA_OK;
 }
 
@@ -648,8 +674,8 @@ int ca_tables_ref(const ca_tables* t, int32_t* final_idx, int32_t* slots, int32_
 }
 
 int ca_tables_plan(const ca_tables* t, ca_work_item* shared_items, ca_work_item* stream_items,
-                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* part_rows,
-                   int32_t* tail_slot, int32_t* tail_fill) {
+                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* tail_slot,
+                   int32_t* tail_fill) {
     if (!t) return fail(CA_ERR_INVALID, "bad argument");
     static_assert(sizeof(ca_work_item) == sizeof(ca::WorkItem), "work item layouts must agree");
     if (shared_items && !t->plan.shared_items.empty()) {
@@ -661,7 +687,6 @@ int ca_tables_plan(const ca_tables* t, ca_work_item* shared_items, ca_work_item*
     copy_i32(slots, t->plan.slots);
     copy_i32(seq_len, t->plan.seq_len);
     copy_i32(part_ptr, t->plan.part_ptr);
-    copy_i32(part_rows, t->plan.part_rows);
     copy_i32(tail_slot, t->plan.tail_slot);
     copy_i32(tail_fill, t->plan.tail_fill);
     return CA_OK;

@@ -22,7 +22,6 @@ struct LaunchArgs {
     const int32_t* slots = nullptr;
     const int32_t* seq_len = nullptr;
     const int32_t* part_ptr = nullptr;
-    const int32_t* part_rows = nullptr;
     int32_t* counters = nullptr;  // [n_seqs * H], zero between launches
     int delta_tokens = 0;
     int H = 0;

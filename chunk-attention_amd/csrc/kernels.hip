@@ -150,8 +150,7 @@ struct DecodeArgs {
     const WorkItem* stream_items;
     const int32_t* slots;
     const int32_t* seq_len;
-    const int32_t* part_ptr;
-    const int32_t* part_rows;
+    const int32_t* part_ptr;  // sequence s owns partial rows part_ptr[s] .. part_ptr[s+1]-1
     int32_t* counters;  // [n_seqs * H] partial rows completed so far, 0 between launches
     int n_shared_wgs;   // workgroups [0, n_shared_wgs) run shared items
     int delta_tokens;
@@ -160,39 +159,48 @@ struct DecodeArgs {
     int fuse_merge;  // 1: the last workgroup to finish a (sequence, head) merges its partials
 };
 
-// Wave-level merge of the partial rows of one (sequence, head): lane l owns output dims
-// 2l, 2l+1.  Maxima and sums are fetched 64 rows at a time, one per lane; the acc rows are
-// then read with independent loads.
-__device__ __forceinline__ void merge_rows(const float* __restrict__ part,
-                                           const int32_t* __restrict__ part_rows, int p0, int p1,
-                                           int h, int H, half_t* __restrict__ out_row, int l) {
-    float m = NEG_INF;
-    for (int p = p0 + l; p < p1; p += 64) {
-        m = fmaxf(m, part_load(part + (size_t(part_rows[p]) * H + h) * PART_STRIDE));
-    }
-    m = wave_max(m);
-    float lsum = 0.f;
+// Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
+// dims 2l, 2l+1.  Rows are taken eight at a time with all their loads in flight together and
+// folded with a running maximum, so a typical merge costs one memory round trip.
+// COHERENT: rows may have been written during this launch by other workgroups (device-scope
+// loads); otherwise they come from an earlier launch and plain loads do.
+template <bool COHERENT>
+__device__ __forceinline__ void merge_rows(const float* __restrict__ part, int p0, int p1, int h,
+                                           int H, half_t* __restrict__ out_row, int l) {
+    float m_run = NEG_INF, lsum = 0.f;
     f2 o = f2{ 0.f, 0.f };
-    for (int pb = p0; pb < p1; pb += 64) {
-        float wp = 0.f;
-        int rowp = 0;
-        if (pb + l < p1) {
-            rowp = part_rows[pb + l];
-            const float* r = part + (size_t(rowp) * H + h) * PART_STRIDE;
-            const float mp = part_load(r);
-            wp = (mp == NEG_INF) ? 0.f : fast_exp2(mp - m);
-            lsum += wp * part_load(r + 1);
+    for (int pb = p0; pb < p1; pb += 8) {
+        f2 ml[8], v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            ml[u] = f2{ NEG_INF, 0.f };
+            v[u] = f2{ 0.f, 0.f };
+            if (pb + u < p1) {
+                const float* r = part + (size_t(pb + u) * H + h) * PART_STRIDE;
+                if constexpr (COHERENT) {
+                    ml[u] = part_load2(r);
+                    v[u] = part_load2(r + 4 + 2 * l);
+                } else {
+                    ml[u] = *reinterpret_cast<const f2*>(r);
+                    v[u] = *reinterpret_cast<const f2*>(r + 4 + 2 * l);
+                }
+            }
         }
-        const int cnt = (p1 - pb < 64) ? (p1 - pb) : 64;
-#pragma unroll 8
-        for (int k = 0; k < cnt; k++) {
-            const float wk = __shfl(wp, k, 64);
-            const int rk = __shfl(rowp, k, 64);
-            const f2 v = part_load2(part + (size_t(rk) * H + h) * PART_STRIDE + 4 + 2 * l);
-            o += wk * v;
+        float mb = m_run;
+#pragma unroll
+        for (int u = 0; u < 8; u++) mb = fmaxf(mb, ml[u][0]);
+        if (mb == NEG_INF) continue;  // nothing but empty rows so far
+        const float fa = (m_run == NEG_INF) ? 0.f : fast_exp2(m_run - mb);
+        o *= fa;
+        lsum *= fa;
+        m_run = mb;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float w = (ml[u][0] == NEG_INF) ? 0.f : fast_exp2(ml[u][0] - mb);
+            o += w * v[u];
+            lsum += w * ml[u][1];
         }
     }
-    lsum = wave_sum(lsum);
     const float r = lsum > 0.f ? 1.f / lsum : 0.f;
     *reinterpret_cast<h2*>(out_row + 2 * l) = h2{ half_t(o[0] * r), half_t(o[1] * r) };
 }
@@ -209,6 +217,7 @@ struct SharedPathLds {
     float m[NW][MROWS];
     float l[NW][MROWS];
     int last[MROWS];
+    int row[MROWS];  // partial row of each covered sequence
 };
 struct StreamPathLds {
     float p[NW][64];
@@ -253,8 +262,9 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
     // is published and nothing remains to merge.  Each wave tries once after its first tile,
     // when the row loads hide behind the streaming; the rest happens at the end.
     const bool can_fold = A.fuse_merge && it.part_row >= 0;
-    const int p0 = can_fold ? A.part_ptr[seq] : 0;
-    const int p1 = can_fold ? A.part_ptr[seq + 1] : 0;
+    const int p0 = (it.part_row >= 0) ? A.part_ptr[seq] : 0;
+    const int p1 = (it.part_row >= 0) ? A.part_ptr[seq + 1] : 0;
+    const int own = p0 + it.part_row;  // this workgroup's partial row
     int* counter = A.counters + (seq * H + h);
     bool folded = !can_fold;
     auto fold_rows = [&]() {
@@ -267,9 +277,8 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
                 const int p = pb + u * NW;
                 rm[u] = NEG_INF;
                 rl[u] = 0.f;
-                const int row = (p < p1) ? A.part_rows[p] : it.part_row;
-                if (row != it.part_row) {
-                    const float* r = A.part + (size_t(row) * H + h) * PART_STRIDE;
+                if (p < p1 && p != own) {
+                    const float* r = A.part + (size_t(p) * H + h) * PART_STRIDE;
                     const f2 ml = part_load2(r);
                     rm[u] = ml[0];
                     rl[u] = ml[1];
@@ -419,7 +428,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
         if (complete && tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
-    float* own_row = A.part + (size_t(it.part_row) * H + h) * PART_STRIDE;
+    float* own_row = A.part + (size_t(own) * H + h) * PART_STRIDE;
     if (tid < D) part_store(own_row + 4 + tid, o);
     if (tid == 0) part_store2(own_row, m, lsum);
     if (!A.fuse_merge) return;
@@ -433,7 +442,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
     }
     __syncthreads();
     if (sm.state && w == 0) {
-        merge_rows(A.part, A.part_rows, p0, p1, h, H, A.out + (size_t(seq) * H + h) * D, l);
+        merge_rows<true>(A.part, p0, p1, h, H, A.out + (size_t(seq) * H + h) * D, l);
         if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -463,6 +472,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
     const int len = A.seq_len[it.len_seq] + A.delta_tokens;
     const bool two = it.n_rows > 16;  // second 16-row block in use (uniform)
+    if (tid < it.n_rows) sm.row[tid] = A.part_ptr[it.seq_begin + tid] + it.part_row;
 
     // Q^T operand: sequence row mb*16+i, dims 32*ks + 8*g .. +7
     h8 qreg[MB][4];
@@ -617,7 +627,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     // ---- write the partial rows ------------------------------------------------------------
     for (int idx = tid; idx < it.n_rows * (D / 4); idx += WG) {
         const int row = idx / (D / 4), c4 = idx % (D / 4);
-        float* dst = A.part + (size_t(it.part_row + row) * H + h) * PART_STRIDE + 4 + 4 * c4;
+        float* dst = A.part + (size_t(sm.row[row]) * H + h) * PART_STRIDE + 4 + 4 * c4;
         const f4 v = *reinterpret_cast<const f4*>(&sm.o[row * OPITCH + 4 * c4]);
         part_store2(dst, v[0], v[1]);
         part_store2(dst + 2, v[2], v[3]);
@@ -630,7 +640,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
                 float lsum = 0.f;
 #pragma unroll
                 for (int k = 0; k < NW; k++) lsum += sm.l[k][row];
-                part_store2(A.part + (size_t(it.part_row + row) * H + h) * PART_STRIDE, m_all[mb], lsum);
+                part_store2(A.part + (size_t(sm.row[row]) * H + h) * PART_STRIDE, m_all[mb], lsum);
             }
         }
     }
@@ -649,8 +659,8 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     for (int r = w; r < it.n_rows; r += NW) {
         if (sm.last[r]) {
             const int s = it.seq_begin + r;
-            merge_rows(A.part, A.part_rows, A.part_ptr[s], A.part_ptr[s + 1], h, H,
-                       A.out + (size_t(s) * H + h) * D, l);
+            merge_rows<true>(A.part, A.part_ptr[s], A.part_ptr[s + 1], h, H,
+                             A.out + (size_t(s) * H + h) * D, l);
             if (l == 0) __hip_atomic_store(&A.counters[s * H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -677,7 +687,6 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
 __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ part,
                                                    half_t* __restrict__ out,
                                                    const int32_t* __restrict__ part_ptr,
-                                                   const int32_t* __restrict__ part_rows,
                                                    int n_seqs, int H) {
     const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
     const int sh = blockIdx.x * NW + w;
@@ -685,7 +694,7 @@ __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ par
     const int seq = sh / H, h = sh % H;
     const int p0 = part_ptr[seq], p1 = part_ptr[seq + 1];
     if (p0 == p1) return;  // written directly by a stream item
-    merge_rows(part, part_rows, p0, p1, h, H, out + (size_t(seq) * H + h) * D, l);
+    merge_rows<false>(part, p0, p1, h, H, out + (size_t(seq) * H + h) * D, l);
 }
 
 __global__ __launch_bounds__(WG) void fill_kernel(int32_t* __restrict__ p, int n, int32_t value) {
@@ -757,7 +766,6 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.slots = a.slots;
     d.seq_len = a.seq_len;
     d.part_ptr = a.part_ptr;
-    d.part_rows = a.part_rows;
     d.counters = a.counters;
     d.n_shared_wgs = 0;
     d.delta_tokens = a.delta_tokens;
@@ -789,7 +797,7 @@ int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st) {
     if (n_seqs <= 0) return 0;
     const int waves = n_seqs * a.H;
     hipLaunchKernelGGL(merge_kernel, dim3((waves + NW - 1) / NW), dim3(WG), 0, st, a.part,
-                       static_cast<half_t*>(a.out), a.part_ptr, a.part_rows, n_seqs, a.H);
+                       static_cast<half_t*>(a.out), a.part_ptr, n_seqs, a.H);
     CA_LAUNCH_CHECK();
     return 0;
 }

@@ -107,15 +107,15 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     }
     int seg_chunks = params.shared_seg_chunks;
     if (seg_chunks <= 0) {
-        // aim at about one workgroup per compute unit, but keep segments between 1 and 16
-        // chunks: the shared workgroups then leave room for streaming ones from the start, and
-        // longer segments mean fewer partial rows to write and merge
-        const int64_t target = params.n_cus;
+        // aim at about one workgroup per two compute units, but keep segments between 1 and
+        // 16 chunks: the shared workgroups then leave most slots to streaming ones from the
+        // start, and longer segments mean fewer partial rows to write and merge
+        const int64_t target = std::max(params.n_cus / 2, 1);
         const int64_t wgs_at_1 = shared_units * std::max(params.n_heads, 1);
         seg_chunks = static_cast<int>(std::clamp<int64_t>(wgs_at_1 / std::max<int64_t>(target, 1), 1, 16));
     }
 
-    std::vector<std::vector<int32_t>> parts_of_seq(n_seqs);
+    std::vector<int32_t> n_parts(n_seqs, 0);  // partial rows handed out per sequence so far
     for (const Run& run : runs) {
         const ChunkRow& r0 = rows[run.first_row];
         const int n = r0.seq_end - r0.seq_begin;
@@ -129,16 +129,22 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 p.slots.push_back(rows[run.first_row + k].slot);
                 p.shared_tokens += rows[run.first_row + k].n_tokens;
             }
-            const int part_base = p.n_part_rows;
-            p.n_part_rows += n;
-            for (int s = 0; s < n; s++) parts_of_seq[r0.seq_begin + s].push_back(part_base + s);
+            // every covered sequence has the same chunks above this one, so this segment is
+            // the same ordinal among the partial rows of each of them
+            const int ordinal = n_parts[r0.seq_begin];
+            for (int s = 0; s < n; s++) {
+                if (n_parts[r0.seq_begin + s] != ordinal) {
+                    throw std::logic_error("tables: sequences of one shared chunk disagree on its position");
+                }
+                n_parts[r0.seq_begin + s]++;
+            }
             for (int m0 = 0; m0 < n; m0 += kMaxRows) {
                 WorkItem it{};
                 it.seq_begin = r0.seq_begin + m0;
                 it.n_rows = std::min(kMaxRows, n - m0);
                 it.slot_first = slot_first;
                 it.n_chunks = c1 - c0;
-                it.part_row = part_base + m0;
+                it.part_row = ordinal;
                 it.pos0 = pos[run.first_row + c0];
                 it.len_seq = r0.seq_begin;
                 p.shared_items.push_back(it);
@@ -195,8 +201,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 p.slots.push_back(rows[own[k]].slot);
                 p.stream_tokens += rows[own[k]].n_tokens;
             }
-            it.part_row = p.n_part_rows++;
-            parts_of_seq[s].push_back(it.part_row);
+            it.part_row = n_parts[s]++;
             p.stream_items.push_back(it);
         }
     }
@@ -204,19 +209,18 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     // a sequence whose only partial comes from a stream item needs no merge: that item
     // writes the final output itself and its partial row is dropped from the merge list
     for (auto& it : p.stream_items) {
-        auto& parts = parts_of_seq[it.seq_begin];
-        if (parts.size() == 1) {
+        if (n_parts[it.seq_begin] == 1) {
             it.part_row = -1;
-            parts.clear();
+            n_parts[it.seq_begin] = 0;
         }
     }
 
     p.part_ptr.assign(n_seqs + 1, 0);
     for (int s = 0; s < n_seqs; s++) {
-        p.part_ptr[s + 1] = p.part_ptr[s] + static_cast<int>(parts_of_seq[s].size());
-        p.max_parts_per_seq = std::max(p.max_parts_per_seq, static_cast<int>(parts_of_seq[s].size()));
-        p.part_rows.insert(p.part_rows.end(), parts_of_seq[s].begin(), parts_of_seq[s].end());
+        p.part_ptr[s + 1] = p.part_ptr[s] + n_parts[s];
+        p.max_parts_per_seq = std::max(p.max_parts_per_seq, n_parts[s]);
     }
+    p.n_part_rows = p.part_ptr[n_seqs];
 }
 
 }  // namespace ca

@@ -42,7 +42,9 @@ struct WorkItem {
     int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared)
     int32_t slot_first;  // index into Plan::slots of the item's first chunk
     int32_t n_chunks;    // consecutive entries of Plan::slots
-    int32_t part_row;    // first partial row written; -1: write the final output directly
+    int32_t part_row;    // which of its sequence's partial rows the item writes: row
+                         // part_ptr[seq] + part_row (for every covered sequence of a shared
+                         // item); -1: the item writes the final output directly
     int32_t pos0;        // position of the first chunk on the sequence's root->leaf path
     int32_t len_seq;     // sequence whose length bounds the valid tokens of these chunks
     int32_t reserved;
@@ -71,8 +73,7 @@ struct Plan {
     std::vector<WorkItem> stream_items;
     std::vector<int32_t> slots;      // chunk slot lists the items index into
     std::vector<int32_t> seq_len;    // tokens per sequence when the plan was built
-    std::vector<int32_t> part_ptr;   // [n_seqs + 1] CSR into part_rows
-    std::vector<int32_t> part_rows;  // partial rows to merge, per sequence
+    std::vector<int32_t> part_ptr;   // [n_seqs + 1]: sequence s owns partial rows part_ptr[s] .. part_ptr[s+1]
     std::vector<int32_t> tail_slot;  // per sequence: slot of its last chunk
     std::vector<int32_t> tail_fill;  // per sequence: tokens in that chunk when built
 };

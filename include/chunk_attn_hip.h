@@ -108,12 +108,19 @@ int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
  * reference's partial buffers. */
 int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
 
+/* How ca_attention is launched.  0 (default): one launch in which chunk-first and sequence-
+ * first workgroups run side by side and write partial rows, then a merge launch.  1: a single
+ * launch in which the workgroup that finishes the last partial of a (sequence, head) merges
+ * them (completion counters; usually slower, kept for callers that need one launch). */
+int ca_ctx_set_schedule(ca_ctx* ctx, int mode);
+
 /* Timing of ca_attention with HIP events recorded on the stream the kernels are launched on
  * (the reference marks its phases with NVTX ranges, kernel_cuda.cu:1334-1433).
- * mode 0: off.  mode 1: every ca_attention call is bracketed by two events; ca_ctx_read_timing
- * returns the accumulated milliseconds of the fused launch in *shared_ms (the other two stay 0).
- * mode 2: ca_attention runs as three separately timed launches (chunk-first, sequence-first,
- * merge) and the three accumulators are filled; for phase analysis, slower than the fused launch. */
+ * mode 0: off.  mode 1: ca_attention runs as it normally does with events around its launches;
+ * ca_ctx_read_timing returns the accumulated milliseconds of the decode launch in *shared_ms
+ * and of the merge launch in *merge_ms (*stream_ms stays 0).  mode 2: ca_attention runs as
+ * three separately timed launches (chunk-first, sequence-first, merge) and the three
+ * accumulators are filled; for phase analysis, slower than the normal forward. */
 int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
@@ -169,16 +176,17 @@ int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n
 void ca_tables_destroy(ca_tables* t);
 /* sizes: fills the same struct ca_ctx_plan_info fills */
 int ca_tables_info(const ca_tables* t, ca_plan_info* info);
-/* lengths of the variable-size plan arrays: n_slots, n_part_list */
-int ca_tables_plan_sizes(const ca_tables* t, int* n_slots, int* n_part_list);
+/* length of the plan's slot list */
+int ca_tables_plan_sizes(const ca_tables* t, int* n_slots);
 /* reference-form tables, same buffers as ca_ctx_ref_tables */
 int ca_tables_ref(const ca_tables* t, int32_t* final_idx, int32_t* slots, int32_t* begins,
                   int32_t* ends, int32_t* offsets, int32_t* seq_n_tokens, int32_t* seq_chunk_map);
 /* packed plan: shared_items [n_shared_items], stream_items [n_stream_items], slots [n_slots],
- * seq_len / tail_slot / tail_fill [n_seqs], part_ptr [n_seqs + 1], part_rows [n_part_list] */
+ * seq_len / tail_slot / tail_fill [n_seqs], part_ptr [n_seqs + 1] (sequence s owns partial
+ * rows part_ptr[s] .. part_ptr[s+1]-1; an item writes row part_ptr[seq] + item.part_row) */
 int ca_tables_plan(const ca_tables* t, ca_work_item* shared_items, ca_work_item* stream_items,
-                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* part_rows,
-                   int32_t* tail_slot, int32_t* tail_fill);
+                   int32_t* slots, int32_t* seq_len, int32_t* part_ptr, int32_t* tail_slot,
+                   int32_t* tail_fill);
 
 /* ---- prefix-tree chunk manager -------------------------------------------------------- */
 

@@ -44,22 +44,25 @@ def check_plan(rows, n_seqs, c, plan, tpp, partition):
     """Every (sequence, chunk) pair is attended exactly once, in path order; partial lists
     name exactly the rows the items write."""
     covered = {s: [] for s in range(n_seqs)}        # s -> list of (pos, slot)
-    written = {}                                    # part_row -> seq
+    written = {}                                    # absolute part row -> seq
     slots = plan["slots"]
+    pp = plan["part_ptr"]
     for it in plan["shared_items"]:
         b, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
-        assert 1 <= n <= 64 and nc >= 1
+        assert 1 <= n <= 32 and nc >= 1 and pr >= 0
         for i in range(n):
-            assert pr + i not in written
-            written[pr + i] = b + i
+            row = int(pp[b + i]) + pr
+            assert row not in written
+            written[row] = b + i
             for k in range(nc):
                 covered[b + i].append((pos0 + k, int(slots[sf + k])))
     for it in plan["stream_items"]:
         s, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
         assert n == 1 and lseq == s and nc >= 1
         if pr >= 0:
-            assert pr not in written
-            written[pr] = s
+            row = int(pp[s]) + pr
+            assert row not in written
+            written[row] = s
         for k in range(nc):
             covered[s].append((pos0 + k, int(slots[sf + k])))
     # expected coverage from the rows
@@ -71,17 +74,18 @@ def check_plan(rows, n_seqs, c, plan, tpp, partition):
             depth[s] += 1
     for s in range(n_seqs):
         assert sorted(covered[s]) == want[s]
-        lst = plan["part_rows"][plan["part_ptr"][s]:plan["part_ptr"][s + 1]].tolist()
+        lst = list(range(int(pp[s]), int(pp[s + 1])))       # the rows the merge reads
         mine = sorted(r for r, q in written.items() if q == s)
         direct = [it for it in plan["stream_items"] if it[0] == s and it[4] < 0]
         if direct:
             assert lst == [] and mine == [] and len(direct) == 1
         else:
-            assert sorted(lst) == mine and len(mine) >= 1
+            assert lst == mine and len(mine) >= 1
         assert plan["seq_len"][s] == sum(nt for (_, nt, b, e) in rows.tolist() if b <= s < e)
         last = [r for r in rows.tolist() if r[2] <= s < r[3]][-1]
         assert (plan["tail_slot"][s], plan["tail_fill"][s]) == (last[0], last[1])
     assert all(0 <= r < plan["n_part_rows"] for r in written)
+    assert plan["n_part_rows"] == int(pp[n_seqs]) == len(written)
     if partition == 2:
         assert len(plan["shared_items"]) == 0
     if partition == 1:
