@@ -242,7 +242,7 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
                  n_heads: int = 32, n_cus: int = 256) -> dict:
     """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
     (work items as [n, 8] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
-    len_seq, reserved; an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
+    len_seq, flags (1 = wide shared item); an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
     lib = load()
     rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
     h = ctypes.c_void_p()

@@ -383,6 +383,12 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
             if (int rc = build_and_upload(c, partition, st)) return rc;
         }
         if (!c->timing) return run_fused(c, q, out, st);
+        if (c->timing == 3) {
+            // measurement aid: only the decode launch, so that a caller can time a train of them
+            const ca::LaunchArgs a3 = launch_args(c, q, out);
+            return launch_rc(ca::launch_decode(a3, static_cast<int>(c->plan.shared_items.size()),
+                                               static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
+        }
         if (int rc = collect_timing(c)) return rc;
         CA_HIP(hipEventRecord(c->ev[0], st));
         if (c->timing == 1 && c->schedule == 0) {
@@ -415,7 +421,7 @@ int ca_ctx_set_timing(ca_ctx* c, int enable) {
     if (enable && !c->ev[0]) {
         for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
     }
-    if (enable < 0 || enable > 2) return fail(CA_ERR_INVALID, "timing mode must be 0, 1 or 2");
+    if (enable < 0 || enable > 3) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2 or 3");
     if (int rc = collect_timing(c)) return rc;
     c->timing = enable;
     return CA_OK;

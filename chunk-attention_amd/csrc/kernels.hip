@@ -226,9 +226,17 @@ struct StreamPathLds {
     float l[NW];
     int state;  // workgroup-uniform decision flags
 };
+constexpr int KPITCH = D + 8;   // halves per LDS row of a K tile (272 B: rows stay 16-byte aligned)
+constexpr int WROWS = 4 * MROWS;  // sequences per wide item: 32 per wave
+struct WidePathLds {
+    half_t k[64 * KPITCH];
+    half_t v[64 * VPITCH];
+    int last[WROWS];
+};
 union __attribute__((aligned(16))) DecodeLds {
     SharedPathLds sh;
     StreamPathLds st;
+    WidePathLds wd;
 };
 
 template <int C>
@@ -666,6 +674,199 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// wide_path: chunk-first for chunks shared by many sequences.  An item covers up to 128
+// sequences; wave w owns rows 32w .. 32w+31 (Q^T and the output accumulators stay in its
+// registers for the whole segment) and attends every token.  The segment is walked in 64-token
+// tiles: all 256 threads stage the K and V tile in LDS once (the next tile is already on its way
+// in registers), then each wave runs the same MFMA scheme as shared_path with K operands read
+// from LDS.  Every K/V byte is fetched once per 128 sequences and no cross-wave merge is needed.
+// ---------------------------------------------------------------------------------------
+template <int C>
+__device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem& it, int h,
+                                          WidePathLds& sm) {
+    const half_t* __restrict__ kpool = A.kpool;
+    const half_t* __restrict__ vpool = A.vpool;
+    const int32_t* __restrict__ slots = A.slots;
+    const int H = A.H;
+    const float scale_log2 = A.scale_log2;
+    const int tid = threadIdx.x;
+    const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
+    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
+    const int row_base = 32 * w;                    // first item row of this wave
+    const bool active = row_base < it.n_rows;       // wave has sequences (uniform per wave)
+    const bool two = row_base + 16 < it.n_rows;
+
+    h8 qreg[MB][4];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        const int row = row_base + mb * 16 + i;
+        const half_t* qp = A.q + (size_t(it.seq_begin + row) * H + h) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
+        }
+    }
+    float m_run[MB], l_lane[MB];
+    f4 oacc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        m_run[mb] = NEG_INF;
+        l_lane[mb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < 8; db++) oacc[mb][db] = f4{ 0.f, 0.f, 0.f, 0.f };
+    }
+
+    // tile t = tokens 64t .. 64t+63 of the segment.  Thread tid stages pieces tid + 256r
+    // (r = 0..3) of the K and of the V tile: piece p = row p/16, dims 8*(p%16) .. +7.
+    const int total_tokens = it.n_chunks * C;
+    const int n_tiles = (total_tokens + 63) / 64;
+    uint4 kst[4], vst[4];
+    auto fetch_tile = [&](int t) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int p = tid + 256 * r;
+            const int tok = 64 * t + (p >> 4);  // token of the segment
+            const int ck = tok / C;
+            const int valid = len - (it.pos0 + ck) * C - (tok % C);  // > 0: token exists
+            if (tok < total_tokens && valid > 0) {
+                const size_t off = ((size_t(slots[it.slot_first + ck]) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
+                kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
+                vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
+            } else {
+                kst[r] = make_uint4(0, 0, 0, 0);  // missing tokens: zero V, scores masked below
+                vst[r] = make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    // number of existing tokens in tile t (tokens exist as a prefix of the segment)
+    auto tile_valid = [&](int t) {
+        int have = len - it.pos0 * C - 64 * t;
+        const int cap = total_tokens - 64 * t;
+        have = have < cap ? have : cap;
+        return have < 64 ? have : 64;
+    };
+
+    if (n_tiles > 0) fetch_tile(0);
+    for (int t = 0; t < n_tiles; t++) {
+        const int valid = tile_valid(t);
+        if (valid <= 0) break;  // uniform: nothing further exists
+        __syncthreads();        // everyone is done reading the previous tile
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int p = tid + 256 * r;
+            *reinterpret_cast<uint4*>(&sm.k[(p >> 4) * KPITCH + 8 * (p & 15)]) = kst[r];
+            uint2* dv = reinterpret_cast<uint2*>(&sm.v[(p >> 4) * VPITCH + 8 * (p & 15)]);
+            dv[0] = make_uint2(vst[r].x, vst[r].y);
+            dv[1] = make_uint2(vst[r].z, vst[r].w);
+        }
+        __syncthreads();
+        if (t + 1 < n_tiles) fetch_tile(t + 1);
+        if (!active) continue;
+
+        // scores of the 64 tokens for this wave's rows
+        f4 sc[MB][4];
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) {
+            h8 kop[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                kop[ks] = *reinterpret_cast<const h8*>(&sm.k[(16 * tb + i) * KPITCH + 32 * ks + 8 * g]);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                f4 acc = f4{ 0.f, 0.f, 0.f, 0.f };
+                if (mb == 0 || two) {
+#pragma unroll
+                    for (int ks = 0; ks < 4; ks++) {
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[ks], qreg[mb][ks], acc, 0, 0, 0);
+                    }
+                }
+                sc[mb][tb] = acc;
+            }
+        }
+        h4 pb[MB][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            float mx = NEG_INF;
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float v = (16 * tb + 4 * g + r < valid) ? sc[mb][tb][r] * scale_log2 : NEG_INF;
+                    sc[mb][tb][r] = v;
+                    mx = fmaxf(mx, v);
+                }
+            }
+            mx = fmaxf(mx, shfl_xor(mx, 16));
+            mx = fmaxf(mx, shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run[mb], mx);
+            const float alpha = fast_exp2(m_run[mb] - m_new);
+            m_run[mb] = m_new;
+            float psum = 0.f;
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++) {
+                float p[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    p[r] = fast_exp2(sc[mb][tb][r] - m_new);
+                    psum += p[r];
+                }
+                pb[mb][tb] = h4{ half_t(p[0]), half_t(p[1]), half_t(p[2]), half_t(p[3]) };
+            }
+            l_lane[mb] = l_lane[mb] * alpha + psum;
+#pragma unroll
+            for (int db = 0; db < 8; db++) oacc[mb][db] *= alpha;
+        }
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int db = 0; db < 8; db++) {
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++) {
+                const half_t* col = &sm.v[(16 * tb + 4 * g) * VPITCH + 16 * db + i];
+                const h4 a = h4{ col[0], col[VPITCH], col[2 * VPITCH], col[3 * VPITCH] };
+                oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[0][tb], oacc[0][db], 0, 0, 0);
+                if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1][tb], oacc[1][db], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- each wave writes the partial rows of its own sequences ----------------------------
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        l_lane[mb] += shfl_xor(l_lane[mb], 16);
+        l_lane[mb] += shfl_xor(l_lane[mb], 32);
+        const int row = row_base + mb * 16 + i;
+        if (row < it.n_rows) {
+            float* dst = A.part + (size_t(A.part_ptr[it.seq_begin + row] + it.part_row) * H + h) * PART_STRIDE;
+            if (g == 0) part_store2(dst, m_run[mb], l_lane[mb]);
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                part_store2(dst + 4 + 16 * db + 4 * g, oacc[mb][db][0], oacc[mb][db][1]);
+                part_store2(dst + 4 + 16 * db + 4 * g + 2, oacc[mb][db][2], oacc[mb][db][3]);
+            }
+        }
+    }
+    if (!A.fuse_merge) return;
+
+    wait_own_stores();
+    __syncthreads();
+    for (int r = tid; r < it.n_rows; r += WG) {
+        const int s = it.seq_begin + r;
+        const int done = __hip_atomic_fetch_add(&A.counters[s * H + h], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sm.last[r] = (done == A.part_ptr[s + 1] - A.part_ptr[s] - 1);
+    }
+    __syncthreads();
+    for (int r = w; r < it.n_rows; r += NW) {
+        if (sm.last[r]) {
+            const int s = it.seq_begin + r;
+            merge_rows<true>(A.part, A.part_ptr[s], A.part_ptr[s + 1], h, H,
+                             A.out + (size_t(s) * H + h) * D, l);
+            if (l == 0) __hip_atomic_store(&A.counters[s * H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // grid = (n_shared_items + n_stream_items) * H workgroups, shared items first: they have the
 // longest dependent chains and are sized to about one per compute unit, so they are done long
 // before the streaming is and the merge falls to stream workgroups, one row each.
@@ -675,7 +876,11 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
     const int bid = blockIdx.x;
     if (bid < A.n_shared_wgs) {
         const WorkItem it = A.shared_items[bid / A.H];
-        shared_path<C>(A, it, bid % A.H, lds.sh);
+        if (it.flags & kItemWide) {
+            wide_path<C>(A, it, bid % A.H, lds.wd);
+        } else {
+            shared_path<C>(A, it, bid % A.H, lds.sh);
+        }
     } else {
         const int sid = bid - A.n_shared_wgs;
         const WorkItem it = A.stream_items[sid / A.H];

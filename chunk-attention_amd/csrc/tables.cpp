@@ -52,6 +52,7 @@ void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_si
 
 namespace {
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
+int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 }  // namespace
 
 void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
@@ -102,17 +103,29 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             j++;
         }
         runs.push_back({ i, j - i });
-        shared_units += int64_t(j - i) * ceil_div(rows[i].seq_end - rows[i].seq_begin, kMaxRows);
+        const int n_run = rows[i].seq_end - rows[i].seq_begin;
+        shared_units += int64_t(j - i) * ceil_div(n_run, n_run >= kWideMin ? kWideRows : kMaxRows);
         i = j;
     }
     int seg_chunks = params.shared_seg_chunks;
     if (seg_chunks <= 0) {
-        // aim at about one workgroup per two compute units, but keep segments between 1 and
-        // 16 chunks: the shared workgroups then leave most slots to streaming ones from the
-        // start, and longer segments mean fewer partial rows to write and merge
-        const int64_t target = std::max(params.n_cus / 2, 1);
-        const int64_t wgs_at_1 = shared_units * std::max(params.n_heads, 1);
-        seg_chunks = static_cast<int>(std::clamp<int64_t>(wgs_at_1 / std::max<int64_t>(target, 1), 1, 16));
+        // A shared workgroup is a dependent chain (a few microseconds per 64 tokens), so a
+        // segment is kept to 512 tokens -- 256 when the whole step is short -- which lets it
+        // finish within the first round of streaming workgroups.  Only when that would make
+        // far more workgroups than the device holds are segments lengthened (fewer partial
+        // rows to write and merge), up to 16 chunks.
+        int64_t all_tokens = 0;
+        for (int i = 0; i < n_rows; i++) {
+            all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
+        }
+        const double step_us = double(all_tokens) * 4.0 * std::max(params.n_heads, 1) * 128.0 / 6.4e6;
+        const int seg_tokens = step_us >= 40.0 ? 512 : 256;
+        seg_chunks = std::max(1, seg_tokens / chunk_size);
+        const int64_t limit = int64_t(8) * params.n_cus;
+        while (seg_chunks < 16 && ceil_div64(shared_units, seg_chunks) * std::max(params.n_heads, 1) > limit) {
+            seg_chunks *= 2;
+        }
+        seg_chunks = std::min(seg_chunks, 16);
     }
 
     std::vector<int32_t> n_parts(n_seqs, 0);  // partial rows handed out per sequence so far
@@ -138,10 +151,13 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 }
                 n_parts[r0.seq_begin + s]++;
             }
-            for (int m0 = 0; m0 < n; m0 += kMaxRows) {
+            const bool wide = n >= kWideMin;
+            const int tile_rows = wide ? kWideRows : kMaxRows;
+            for (int m0 = 0; m0 < n; m0 += tile_rows) {
                 WorkItem it{};
+                it.flags = wide ? kItemWide : 0;
                 it.seq_begin = r0.seq_begin + m0;
-                it.n_rows = std::min(kMaxRows, n - m0);
+                it.n_rows = std::min(tile_rows, n - m0);
                 it.slot_first = slot_first;
                 it.n_chunks = c1 - c0;
                 it.part_row = ordinal;

@@ -39,7 +39,8 @@ void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_si
 // One unit of kernel work: 8 x int32 so that a wave reads it with one 32-byte scalar load.
 struct WorkItem {
     int32_t seq_begin;   // first sequence (row of q) this item attends for
-    int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared)
+    int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared,
+                         // <= kWideRows for wide shared items)
     int32_t slot_first;  // index into Plan::slots of the item's first chunk
     int32_t n_chunks;    // consecutive entries of Plan::slots
     int32_t part_row;    // which of its sequence's partial rows the item writes: row
@@ -47,7 +48,7 @@ struct WorkItem {
                          // item); -1: the item writes the final output directly
     int32_t pos0;        // position of the first chunk on the sequence's root->leaf path
     int32_t len_seq;     // sequence whose length bounds the valid tokens of these chunks
-    int32_t reserved;
+    int32_t flags;       // kItemWide: shared item in the row-split form (up to kWideRows sequences)
 };
 static_assert(sizeof(WorkItem) == 32, "WorkItem must stay 32 bytes");
 
@@ -61,7 +62,10 @@ struct PlanParams {
     int n_cus = 256;
 };
 
-constexpr int kMaxRows = 32;  // sequences per shared work item (M tile)
+constexpr int kMaxRows = 32;    // sequences per shared work item (M tile)
+constexpr int kWideRows = 128;  // sequences per wide shared work item
+constexpr int kWideMin = 96;    // chunks covering at least this many sequences use wide items
+constexpr int32_t kItemWide = 1;
 
 struct Plan {
     int n_seqs = 0;

@@ -120,7 +120,10 @@ int ca_ctx_set_schedule(ca_ctx* ctx, int mode);
  * ca_ctx_read_timing returns the accumulated milliseconds of the decode launch in *shared_ms
  * and of the merge launch in *merge_ms (*stream_ms stays 0).  mode 2: ca_attention runs as
  * three separately timed launches (chunk-first, sequence-first, merge) and the three
- * accumulators are filled; for phase analysis, slower than the normal forward. */
+ * accumulators are filled; for phase analysis, slower than the normal forward.  mode 3:
+ * ca_attention issues only the decode launch (no merge: sequences with more than one partial
+ * get no output) and records nothing, so that a caller can time a back-to-back train of that
+ * launch between two events of its own. */
 int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
@@ -167,7 +170,7 @@ typedef struct ca_tables ca_tables;
 
 /* One unit of kernel work (see csrc/tables.h). */
 typedef struct ca_work_item {
-    int32_t seq_begin, n_rows, slot_first, n_chunks, part_row, pos0, len_seq, reserved;
+    int32_t seq_begin, n_rows, slot_first, n_chunks, part_row, pos0, len_seq, flags;
 } ca_work_item;
 
 int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,

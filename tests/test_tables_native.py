@@ -49,7 +49,7 @@ def check_plan(rows, n_seqs, c, plan, tpp, partition):
     pp = plan["part_ptr"]
     for it in plan["shared_items"]:
         b, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
-        assert 1 <= n <= 32 and nc >= 1 and pr >= 0
+        assert 1 <= n <= (128 if it[7] & 1 else 32) and nc >= 1 and pr >= 0
         for i in range(n):
             row = int(pp[b + i]) + pr
             assert row not in written
