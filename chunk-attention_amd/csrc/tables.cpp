@@ -52,7 +52,6 @@ void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_si
 
 namespace {
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
-int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 }  // namespace
 
 void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
@@ -94,7 +93,6 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     // ---- shared runs -> segments ---------------------------------------------------------
     struct Run { int first_row, count; };
     std::vector<Run> runs;
-    int64_t shared_units = 0;  // (chunk, M tile) pairs
     for (int i = 0; i < n_rows;) {
         if (!is_shared(rows[i])) { i++; continue; }
         int j = i + 1;
@@ -103,36 +101,32 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             j++;
         }
         runs.push_back({ i, j - i });
-        const int n_run = rows[i].seq_end - rows[i].seq_begin;
-        shared_units += int64_t(j - i) * ceil_div(n_run, n_run >= kWideMin ? kWideRows : kMaxRows);
         i = j;
     }
-    int seg_chunks = params.shared_seg_chunks;
-    if (seg_chunks <= 0) {
-        // A shared workgroup is a dependent chain (a few microseconds per 64 tokens), so a
-        // segment is kept to 512 tokens -- 256 when the whole step is short -- which lets it
-        // finish within the first round of streaming workgroups.  Only when that would make
-        // far more workgroups than the device holds are segments lengthened (fewer partial
-        // rows to write and merge), up to 16 chunks.
-        int64_t all_tokens = 0;
-        for (int i = 0; i < n_rows; i++) {
-            all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
-        }
-        const double step_us = double(all_tokens) * 4.0 * std::max(params.n_heads, 1) * 128.0 / 6.4e6;
-        const int seg_tokens = step_us >= 40.0 ? 512 : 256;
-        seg_chunks = std::max(1, seg_tokens / chunk_size);
-        const int64_t limit = int64_t(8) * params.n_cus;
-        while (seg_chunks < 16 && ceil_div64(shared_units, seg_chunks) * std::max(params.n_heads, 1) > limit) {
-            seg_chunks *= 2;
-        }
-        seg_chunks = std::min(seg_chunks, 16);
+    // Segment length.  A shared workgroup is a dependent chain of about 2 us per 64 tokens
+    // (4 us in the wide form), overlapped with the streaming workgroups of the same launch, so
+    // a segment may take a good part of the step's expected duration (bytes at ~6.4 TB/s) but
+    // not more; longer segments mean fewer partial rows to write and merge, which matters
+    // most when a chunk covers many sequences.
+    int64_t all_tokens = 0;
+    for (int i = 0; i < n_rows; i++) {
+        all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
     }
+    const double step_us = double(all_tokens) * 4.0 * std::max(params.n_heads, 1) * 128.0 / 6.4e6;
+    auto seg_chunks_for = [&](int n_covered) {
+        if (params.shared_seg_chunks > 0) return params.shared_seg_chunks;
+        const bool wide = n_covered >= kWideMin;
+        const double tiles = wide ? 0.5 * step_us / 4.0 : 0.4 * step_us / 2.0;
+        const int n_tiles = std::clamp(static_cast<int>(tiles), 4, 32);  // 64-token tiles
+        return std::max(1, n_tiles * 64 / chunk_size);
+    };
 
     std::vector<int32_t> n_parts(n_seqs, 0);  // partial rows handed out per sequence so far
     for (const Run& run : runs) {
         const ChunkRow& r0 = rows[run.first_row];
         const int n = r0.seq_end - r0.seq_begin;
-        const int n_segs = ceil_div(run.count, seg_chunks);
+        const int seg = seg_chunks_for(n);
+        const int n_segs = std::max(1, (run.count + seg / 2) / seg);  // nearest, not ceiling
         for (int g = 0; g < n_segs; g++) {
             // spread chunks evenly over the segments of a run
             const int c0 = int(int64_t(run.count) * g / n_segs);
