@@ -145,9 +145,9 @@ class Tree:
         self.max_chunks = max_chunks
 
     def __del__(self):
-        if getattr(self, "_h", None) and self._h.value:
-            self._lib.ca_tree_destroy(self._h)
-            self._h = ctypes.c_void_p()
+        h, self._h = getattr(self, "_h", None), None
+        if h is not None and h.value:
+            self._lib.ca_tree_destroy(h)
 
     def add_seq(self, tokens: Sequence[int]) -> Tuple[int, int, List[int]]:
         """Returns (seq_idx, tok_begin, slots): tokens[tok_begin:] need their K/V copied into
@@ -299,9 +299,9 @@ class KernelContext:
         self.n_heads, self.d_head, self.chunk_size = n_heads, d_head, chunk_size
 
     def __del__(self):
-        if getattr(self, "_h", None) and self._h.value:
-            self._lib.ca_ctx_destroy(self._h)
-            self._h = ctypes.c_void_p()
+        h, self._h = getattr(self, "_h", None), None
+        if h is not None and h.value:
+            self._lib.ca_ctx_destroy(h)
 
     def refresh(self, rows: np.ndarray, n_seqs: int, stream: int = 0) -> None:
         rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)

@@ -90,7 +90,7 @@ def test_partials_match_reference_layout():
         np.testing.assert_allclose(attns[sl].reshape(H, nn, 128), o, atol=1e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("n_shared_seqs", [1, 3, 16, 17, 40, 64, 65, 100])
+@pytest.mark.parametrize("n_shared_seqs", [1, 3, 16, 17, 40, 64, 65, 95, 96, 100, 128, 129, 200])
 def test_any_number_of_sharing_sequences(n_shared_seqs):
     # M tiling: row counts that are not multiples of 16 and beyond one 64-row tile
     w = synth.prefix_workload("m-tiles", n_shared_seqs, 64, 192, 70, n_heads=4)
@@ -194,3 +194,56 @@ def test_errors_through_the_c_abi():
     odd.add_seq([1, 2, 3], k, k)
     with pytest.raises(capi.ChunkAttnError, match="unsupported chunk_size 48"):
         odd.forward(to_dev(rand16(rng, 1, 2, 128)))
+
+
+@pytest.mark.parametrize("schedule", [0, 1])
+@pytest.mark.parametrize("case", ["prefix", "two-level", "wide", "ragged-appends"])
+def test_both_launch_schedules(schedule, case):
+    # schedule 0: decode launch + merge launch; 1: single launch, the last finisher merges
+    if case == "prefix":
+        w = synth.prefix_workload("p", 24, 64, 640, 300, n_heads=8)
+    elif case == "two-level":
+        w = synth.two_level_workload("t", 4, 6, 32, 256, 160, 70, n_heads=8)
+    elif case == "wide":
+        w = synth.prefix_workload("w", 150, 64, 384, 40, n_heads=4)
+    else:
+        w = synth.prefix_workload("r", 9, 32, 96, 0, n_heads=4)
+        for s, n in enumerate([1, 31, 32, 33, 64, 65, 100, 5, 127]):
+            w.seqs[s].append(synth.Segment(1_000_000 * (s + 1) + np.arange(n), synth.STREAM_K_UNIQUE + s, synth.STREAM_V_UNIQUE + s))
+    attn, _ = load_workload(w)
+    attn.ctx.set_schedule(schedule)
+    rng = np.random.default_rng(7)
+    for step in range(3):
+        q = rand16(rng, w.n_seqs, w.n_heads, 128)
+        want = oracle_output(attn, q)
+        for partition in (0, 1, 2):
+            for _ in range(2):      # twice: completion counters must come back to zero
+                assert_close(attn.forward(to_dev(q), partition), want)
+        k, v = w.append_kv(step)
+        attn.append_token(w.append_tokens(step), to_dev(k), to_dev(v))
+
+
+def test_forward_under_graph_capture():
+    # with valid tables the forward is kernel launches only: capture it once, replay with new q
+    w = synth.two_level_workload("g", 3, 4, 64, 256, 128, 90, n_heads=8)
+    attn, _ = load_workload(w)
+    rng = np.random.default_rng(8)
+    q = to_dev(rand16(rng, w.n_seqs, w.n_heads, 128))
+    out = torch.empty_like(q)
+    attn.refresh_kernel_context()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, side.cuda_stream)   # warm-up
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, torch.cuda.current_stream().cuda_stream)
+    for _ in range(4):
+        qn = rand16(rng, w.n_seqs, w.n_heads, 128)
+        q.copy_(to_dev(qn))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = attn.forward(q)
+        assert torch.equal(out, eager)
+        assert_close(out, oracle_output(attn, qn))
