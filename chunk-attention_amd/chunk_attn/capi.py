@@ -241,8 +241,8 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
                  partition: int = 0, shared_seg_chunks: int = 0, stream_chunks: int = 0,
                  n_heads: int = 32, n_cus: int = 256) -> dict:
     """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
-    (work items as [n, 8] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
-    len_seq, flags (1 = wide shared item); an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
+    (work items as [n, 16] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
+    len0, flags (1 = wide shared item), 8 inline slots; an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
     lib = load()
     rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
     h = ctypes.c_void_p()
@@ -269,8 +269,8 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
         t["partial_rows"] = info.ref_partial_rows
         t["max_seq_n_chunks"] = info.max_seq_n_chunks
         p = {
-            "shared_items": np.zeros((info.n_shared_items, 8), np.int32),
-            "stream_items": np.zeros((info.n_stream_items, 8), np.int32),
+            "shared_items": np.zeros((info.n_shared_items, 16), np.int32),
+            "stream_items": np.zeros((info.n_stream_items, 16), np.int32),
             "slots": np.zeros(n_slots.value, np.int32),
             "seq_len": np.zeros(info.n_seqs, np.int32),
             "part_ptr": np.zeros(info.n_seqs + 1, np.int32),

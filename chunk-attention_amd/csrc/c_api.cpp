@@ -130,7 +130,6 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.shared_items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_shared);
     a.stream_items = reinterpret_cast<const ca::WorkItem*>(c->dev_blob + c->off_stream);
     a.slots = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_slots);
-    a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
     a.part_ptr = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_part_ptr);
     a.counters = c->counters;
     a.delta_tokens = c->delta_tokens;

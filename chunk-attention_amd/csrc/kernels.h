@@ -20,7 +20,6 @@ struct LaunchArgs {
     const WorkItem* shared_items = nullptr;
     const WorkItem* stream_items = nullptr;
     const int32_t* slots = nullptr;
-    const int32_t* seq_len = nullptr;
     const int32_t* part_ptr = nullptr;
     int32_t* counters = nullptr;  // [n_seqs * H], zero between launches
     int delta_tokens = 0;

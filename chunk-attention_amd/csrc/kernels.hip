@@ -139,6 +139,13 @@ __device__ __forceinline__ float reduce_rows16(float (&v)[NV], int j) {
 // Lane l = 16*g + j reads, for load i, the 16 bytes at offset 1024*i + 16*l of a sub-tile:
 // row 4*i + g, dims 8*j..8*j+7, so every load instruction covers 1 KiB of contiguous memory.
 // ---------------------------------------------------------------------------------------
+// Slot of the k-th chunk of an item: the first ones come with the item, the rest from the list.
+// (`gi` is the item in global memory: indexing a register copy dynamically would spill it.)
+__device__ __forceinline__ int item_slot(const WorkItem* __restrict__ gi, int slot_first,
+                                         const int32_t* __restrict__ slots, int k) {
+    return k < kInlineSlots ? gi->inl[k] : slots[slot_first + k];
+}
+
 // Everything a workgroup needs besides its work item.
 struct DecodeArgs {
     const half_t* q;
@@ -149,7 +156,6 @@ struct DecodeArgs {
     const WorkItem* shared_items;
     const WorkItem* stream_items;
     const int32_t* slots;
-    const int32_t* seq_len;
     const int32_t* part_ptr;  // sequence s owns partial rows part_ptr[s] .. part_ptr[s+1]-1
     int32_t* counters;  // [n_seqs * H] partial rows completed so far, 0 between launches
     int n_shared_wgs;   // workgroups [0, n_shared_wgs) run shared items
@@ -240,8 +246,12 @@ union __attribute__((aligned(16))) DecodeLds {
 };
 
 template <int C>
-__device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem& it, int h,
-                                            StreamPathLds& sm) {
+__device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
+                                            int h, StreamPathLds& sm) {
+    WorkItem it;  // header only: the inline slots are read from global memory where needed
+    it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
+    it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
+    it.len0 = gi->len0; it.flags = gi->flags;
     const half_t* __restrict__ q = A.q;
     const half_t* __restrict__ kpool = A.kpool;
     const half_t* __restrict__ vpool = A.vpool;
@@ -255,7 +265,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
     const int tid = threadIdx.x;
     const int w = tid >> 6, l = tid & 63, g = l >> 4, j = l & 15;
     const int seq = it.seq_begin;
-    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
+    const int len = it.len0 + A.delta_tokens;
 
     const h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
 
@@ -321,7 +331,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
         int valid = len - (it.pos0 + t) * C;
         if (valid <= 0) break;  // chunks are in path order: everything after is empty too
         valid = valid < C ? valid : C;
-        const int slot = slots[it.slot_first + t];
+        const int slot = item_slot(gi, it.slot_first, slots, t);
         const size_t base = (size_t(slot) * H + h) * size_t(C) * D;
 #pragma unroll
         for (int sub = 0; sub < NSUB; sub++) {
@@ -469,8 +479,12 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem&
 //   of the 16 x 128 V block read column-wise.
 // ---------------------------------------------------------------------------------------
 template <int C>
-__device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem& it, int h,
-                                            SharedPathLds& sm) {
+__device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
+                                            int h, SharedPathLds& sm) {
+    WorkItem it;
+    it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
+    it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
+    it.len0 = gi->len0; it.flags = gi->flags;
     const half_t* __restrict__ kpool = A.kpool;
     const half_t* __restrict__ vpool = A.vpool;
     const int32_t* __restrict__ slots = A.slots;
@@ -478,7 +492,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     const float scale_log2 = A.scale_log2;
     const int tid = threadIdx.x;
     const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
-    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
+    const int len = it.len0 + A.delta_tokens;
     const bool two = it.n_rows > 16;  // second 16-row block in use (uniform)
     if (tid < it.n_rows) sm.row[tid] = A.part_ptr[it.seq_begin + tid] + it.part_row;
 
@@ -509,7 +523,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
     // valid tokens of block tb (<= 0: past the end of the sequence), and its element offset
     auto block_valid = [&](int tb) { return len - (it.pos0 + tb / BPC) * C - (tb % BPC) * 16; };
     auto block_base = [&](int tb) {
-        return ((size_t(slots[it.slot_first + tb / BPC]) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
+        return ((size_t(item_slot(gi, it.slot_first, slots, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
     };
     h8 kreg[4], knext[4];
     uint4 vraw[4], vnext[4];
@@ -683,8 +697,12 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem&
 // from LDS.  Every K/V byte is fetched once per 128 sequences and no cross-wave merge is needed.
 // ---------------------------------------------------------------------------------------
 template <int C>
-__device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem& it, int h,
-                                          WidePathLds& sm) {
+__device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
+                                          int h, WidePathLds& sm) {
+    WorkItem it;
+    it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
+    it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
+    it.len0 = gi->len0; it.flags = gi->flags;
     const half_t* __restrict__ kpool = A.kpool;
     const half_t* __restrict__ vpool = A.vpool;
     const int32_t* __restrict__ slots = A.slots;
@@ -692,7 +710,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem& i
     const float scale_log2 = A.scale_log2;
     const int tid = threadIdx.x;
     const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
-    const int len = A.seq_len[it.len_seq] + A.delta_tokens;
+    const int len = it.len0 + A.delta_tokens;
     const int row_base = 32 * w;                    // first item row of this wave
     const bool active = row_base < it.n_rows;       // wave has sequences (uniform per wave)
     const bool two = row_base + 16 < it.n_rows;
@@ -730,7 +748,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem& i
             const int ck = tok / C;
             const int valid = len - (it.pos0 + ck) * C - (tok % C);  // > 0: token exists
             if (tok < total_tokens && valid > 0) {
-                const size_t off = ((size_t(slots[it.slot_first + ck]) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
+                const size_t off = ((size_t(item_slot(gi, it.slot_first, slots, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
                 kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
                 vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
             } else {
@@ -875,16 +893,15 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
     __shared__ DecodeLds lds;
     const int bid = blockIdx.x;
     if (bid < A.n_shared_wgs) {
-        const WorkItem it = A.shared_items[bid / A.H];
-        if (it.flags & kItemWide) {
-            wide_path<C>(A, it, bid % A.H, lds.wd);
+        const WorkItem* gi = A.shared_items + bid / A.H;
+        if (gi->flags & kItemWide) {
+            wide_path<C>(A, gi, bid % A.H, lds.wd);
         } else {
-            shared_path<C>(A, it, bid % A.H, lds.sh);
+            shared_path<C>(A, gi, bid % A.H, lds.sh);
         }
     } else {
         const int sid = bid - A.n_shared_wgs;
-        const WorkItem it = A.stream_items[sid / A.H];
-        stream_path<C>(A, it, sid % A.H, lds.st);
+        stream_path<C>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
     }
 }
 
@@ -969,7 +986,6 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.shared_items = a.shared_items;
     d.stream_items = a.stream_items;
     d.slots = a.slots;
-    d.seq_len = a.seq_len;
     d.part_ptr = a.part_ptr;
     d.counters = a.counters;
     d.n_shared_wgs = 0;

@@ -156,7 +156,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 it.n_chunks = c1 - c0;
                 it.part_row = ordinal;
                 it.pos0 = pos[run.first_row + c0];
-                it.len_seq = r0.seq_begin;
+                it.len0 = p.seq_len[r0.seq_begin];
+                for (int k = 0; k < kInlineSlots && k < c1 - c0; k++) it.inl[k] = p.slots[slot_first + k];
                 p.shared_items.push_back(it);
             }
         }
@@ -206,8 +207,9 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             it.slot_first = static_cast<int>(p.slots.size());
             it.n_chunks = c1 - c0;
             it.pos0 = pos[own[c0]];
-            it.len_seq = s;
+            it.len0 = p.seq_len[s];
             for (int k = c0; k < c1; k++) {
+                if (k - c0 < kInlineSlots) it.inl[k - c0] = rows[own[k]].slot;
                 p.slots.push_back(rows[own[k]].slot);
                 p.stream_tokens += rows[own[k]].n_tokens;
             }

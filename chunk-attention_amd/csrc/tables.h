@@ -36,7 +36,10 @@ struct RefTables {
 void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                       int tpp_threshold, RefTables* out);
 
-// One unit of kernel work: 8 x int32 so that a wave reads it with one 32-byte scalar load.
+// One unit of kernel work: 16 x int32, read with one 64-byte scalar load.  The sequence length
+// and the first chunk slots sit in the item itself so that a workgroup can issue its first K/V
+// loads after a single memory round trip.
+constexpr int kInlineSlots = 8;
 struct WorkItem {
     int32_t seq_begin;   // first sequence (row of q) this item attends for
     int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared,
@@ -47,10 +50,12 @@ struct WorkItem {
                          // part_ptr[seq] + part_row (for every covered sequence of a shared
                          // item); -1: the item writes the final output directly
     int32_t pos0;        // position of the first chunk on the sequence's root->leaf path
-    int32_t len_seq;     // sequence whose length bounds the valid tokens of these chunks
+    int32_t len0;        // tokens (when the tables were built) of the sequence whose length
+                         // bounds the valid tokens of these chunks
     int32_t flags;       // kItemWide: shared item in the row-split form (up to kWideRows sequences)
+    int32_t inl[kInlineSlots];  // slots of the first chunks (same as Plan::slots[slot_first ..])
 };
-static_assert(sizeof(WorkItem) == 32, "WorkItem must stay 32 bytes");
+static_assert(sizeof(WorkItem) == 64, "WorkItem must stay 64 bytes");
 
 struct PlanParams {
     int tpp_threshold = 1;

@@ -170,7 +170,8 @@ typedef struct ca_tables ca_tables;
 
 /* One unit of kernel work (see csrc/tables.h). */
 typedef struct ca_work_item {
-    int32_t seq_begin, n_rows, slot_first, n_chunks, part_row, pos0, len_seq, flags;
+    int32_t seq_begin, n_rows, slot_first, n_chunks, part_row, pos0, len0, flags;
+    int32_t inl[8]; /* slots of the item's first chunks */
 } ca_work_item;
 
 int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,

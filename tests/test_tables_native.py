@@ -48,8 +48,9 @@ def check_plan(rows, n_seqs, c, plan, tpp, partition):
     slots = plan["slots"]
     pp = plan["part_ptr"]
     for it in plan["shared_items"]:
-        b, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
+        b, n, sf, nc, pr, pos0, len0, _ = it.tolist()[:8]
         assert 1 <= n <= (128 if it[7] & 1 else 32) and nc >= 1 and pr >= 0
+        assert len0 == plan["seq_len"][b] and it[8:8 + min(nc, 8)].tolist() == slots[sf:sf + min(nc, 8)].tolist()
         for i in range(n):
             row = int(pp[b + i]) + pr
             assert row not in written
@@ -57,8 +58,9 @@ def check_plan(rows, n_seqs, c, plan, tpp, partition):
             for k in range(nc):
                 covered[b + i].append((pos0 + k, int(slots[sf + k])))
     for it in plan["stream_items"]:
-        s, n, sf, nc, pr, pos0, lseq, _ = it.tolist()
-        assert n == 1 and lseq == s and nc >= 1
+        s, n, sf, nc, pr, pos0, len0, _ = it.tolist()[:8]
+        assert n == 1 and len0 == plan["seq_len"][s] and nc >= 1
+        assert it[8:8 + min(nc, 8)].tolist() == slots[sf:sf + min(nc, 8)].tolist()
         if pr >= 0:
             row = int(pp[s]) + pr
             assert row not in written
