@@ -137,6 +137,8 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.C = c->C;
     a.d = c->d;
     a.scale_log2 = 1.4426950408889634f / std::sqrt(static_cast<float>(c->d));
+    // 256 MiB of Infinity Cache on this part: past twice that per forward, stream around it
+    a.stream_nt = int64_t(c->plan.stream_tokens) * 4 * c->H * c->d > (int64_t(512) << 20);
     return a;
 }
 

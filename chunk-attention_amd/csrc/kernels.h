@@ -27,6 +27,10 @@ struct LaunchArgs {
     int C = 0;
     int d = 128;
     float scale_log2 = 0.f;  // log2(e) / sqrt(d_head)
+    // Read the per-sequence (private) chunks with the non-temporal hint.  Worth it when one
+    // forward streams more than the last-level cache holds: the data cannot be found there
+    // again, and without the hint it only displaces what could be.
+    bool stream_nt = false;
 };
 
 // All return 0, -1 for an unsupported shape, or a positive hipError_t.

@@ -79,6 +79,14 @@ __device__ __forceinline__ f2 part_load2(const float* p) {
     return x.f;
 }
 
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+// 16-byte load with the non-temporal hint: K/V rows are read once and should not displace
+// what the caches hold.
+__device__ __forceinline__ uint4 nt_load16(const uint4* p) {
+    const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 __device__ __forceinline__ float dot8(const h8& a, const h8& b, float acc) {
     acc = __builtin_amdgcn_fdot2(h2{ a[0], a[1] }, h2{ b[0], b[1] }, acc, false);
     acc = __builtin_amdgcn_fdot2(h2{ a[2], a[3] }, h2{ b[2], b[3] }, acc, false);
@@ -163,6 +171,7 @@ struct DecodeArgs {
     int H;
     float scale_log2;
     int fuse_merge;  // 1: the last workgroup to finish a (sequence, head) merges its partials
+    int stream_nt;   // 1: private chunks are read with the non-temporal hint (see LaunchArgs)
 };
 
 // Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
@@ -343,9 +352,9 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
             uint4 kr[NL], vr[NL];
             if (!masked) {
 #pragma unroll
-                for (int i = 0; i < NL; i++) kr[i] = kp[64 * i];
+                for (int i = 0; i < NL; i++) kr[i] = A.stream_nt ? nt_load16(kp + 64 * i) : kp[64 * i];
 #pragma unroll
-                for (int i = 0; i < NL; i++) vr[i] = vp[64 * i];
+                for (int i = 0; i < NL; i++) vr[i] = A.stream_nt ? nt_load16(vp + 64 * i) : vp[64 * i];
             } else {
                 // rows past the end of the sequence hold stale data: never read into the math
 #pragma unroll
@@ -993,6 +1002,7 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.H = a.H;
     d.scale_log2 = a.scale_log2;
     d.fuse_merge = 0;
+    d.stream_nt = a.stream_nt ? 1 : 0;
     return d;
 }
 
