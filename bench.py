@@ -100,6 +100,30 @@ def decode_launch_us(attn, q, out, steps, torch):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
+def side_costs(attn, w, torch, capi):
+    """Per-decode-step costs outside the timed forward: a forced table rebuild (tree walk, plan,
+    upload) and the append kernel, as wall-clock microseconds between device syncs."""
+    import numpy as np
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 20
+    for _ in range(reps):
+        attn.refresh_kernel_context(force=True)
+    torch.cuda.synchronize()
+    refresh_us = (time.perf_counter() - t0) * 1e6 / reps
+    k = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    attn.refresh_kernel_context()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):   # rewrites the same free row of every tail: the cache is not advanced
+        attn.ctx.append_kv(k.data_ptr(), k.data_ptr(), w.n_seqs, stream)
+    torch.cuda.synchronize()
+    append_us = (time.perf_counter() - t0) * 1e6 / reps
+    return {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
+            "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
+
+
 def cpu_baseline(attn, q_np, budget_s, torch):
     """The CPU restatement of the reference's MKL path on the same cache contents (fp16 values
     widened to fp32), timed on this machine's host cores."""
@@ -221,6 +245,8 @@ def main() -> int:
                      "traffic_note": traffic_note,
                      "bytes_per_launch": decode_bytes, "avg_launch_us": round(decode_ms * 1e3, 2)},
     }
+
+    result["per_step_side_costs"] = side_costs(attn, w, torch, capi)
 
     if not args.no_paged:
         pw = synth.paged_variant(w)
