@@ -120,7 +120,28 @@ def side_costs(attn, w, torch, capi):
         attn.ctx.append_kv(k.data_ptr(), k.data_ptr(), w.n_seqs, stream)
     torch.cuda.synchronize()
     append_us = (time.perf_counter() - t0) * 1e6 / reps
+    # the decode step's rotary embedding: as its own launch before the append (the reference's
+    # sequence), and folded into the append launch
+    qr = torch.zeros_like(k)
+    cache = torch.zeros((8192, w.d_head), dtype=torch.float16, device="cuda:0")
+    pos = torch.zeros(w.n_seqs, dtype=torch.int64, device="cuda:0")
+    q2, k2 = qr.view(w.n_seqs, -1), k.view(w.n_seqs, -1)
+    capi.rotary_embedding(pos, q2, k2, w.d_head, cache, True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        capi.rotary_embedding(pos, q2, k2, w.d_head, cache, True)
+        attn.ctx.append_kv(k.data_ptr(), k.data_ptr(), w.n_seqs, stream)
+    torch.cuda.synchronize()
+    two_us = (time.perf_counter() - t0) * 1e6 / reps
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        attn.ctx.rope_append_kv(0, qr.data_ptr(), k.data_ptr(), k.data_ptr(), cache.data_ptr(), 8192, w.d_head,
+                                True, w.n_seqs, stream)
+    torch.cuda.synchronize()
+    fused_us = (time.perf_counter() - t0) * 1e6 / reps
     return {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
+            "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
 
 

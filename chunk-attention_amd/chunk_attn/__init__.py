@@ -10,10 +10,10 @@ import os as _os
 _libdir = _os.path.join(_os.path.dirname(_os.path.abspath(__file__)), "lib")
 try:
     import torch as _torch  # noqa: F401  (loads libtorch before the extension module)
-    from .lib.chunk_attn_c import Attention, Chunk, IntFuture  # noqa: F401
+    from .lib.chunk_attn_c import Attention, Chunk, IntFuture, ops  # noqa: F401
 except ImportError as _e:  # pragma: no cover
     raise ImportError(
         "chunk_attn: the native module is missing or does not load (%s). Build it with "
         "`python chunk-attention_amd/build.py`; the decode path has no fallback." % _e) from _e
 
-__all__ = ["Attention", "Chunk", "IntFuture"]
+__all__ = ["Attention", "Chunk", "IntFuture", "ops"]

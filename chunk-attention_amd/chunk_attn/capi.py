@@ -59,6 +59,13 @@ SIGNATURES = {
                                           ctypes.c_int, ctypes.c_void_p]),
     "ca_append_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                     ctypes.c_void_p]),
+    "ca_rotary_embedding": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                           ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                           ctypes.c_void_p]),
+    "ca_rope_append_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "ca_scatter_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
@@ -233,6 +240,38 @@ class Tree:
         return root
 
 
+def rotary_embedding(positions, query, key, head_size: int, cos_sin_cache, is_neox: bool = True) -> None:
+    """In-place rotary embedding of torch fp16 tensors, the operator the reference exports as
+    `chunk_attn.ops.rotary_embedding` (python_exports_ops.cpp:13): positions int64 [n_tokens] (or
+    [batch, seq]), query [..., n_heads*head_size], key [..., n_kv_heads*head_size], rows
+    contiguous, cos_sin_cache [max_position, rot_dim]."""
+    import torch
+    for name, t in (("query", query), ("key", key), ("cos_sin_cache", cos_sin_cache)):
+        if t.dtype != torch.float16 or t.device.type != "cuda":
+            raise RuntimeError(f"{name} must be an fp16 tensor on the GPU")
+    if positions.dtype != torch.int64 or positions.device != query.device or not positions.is_contiguous():
+        raise RuntimeError("positions must be a contiguous int64 tensor on the query's device")
+    if query.stride(-1) != 1 or key.stride(-1) != 1 or not cos_sin_cache.is_contiguous():
+        raise RuntimeError("query/key rows and cos_sin_cache must be contiguous")
+    n_tokens = query.numel() // query.shape[-1]
+    if positions.numel() != n_tokens or key.numel() // key.shape[-1] != n_tokens:
+        raise RuntimeError("positions, query and key disagree on the number of tokens")
+    if query.shape[-1] % head_size or key.shape[-1] % head_size:
+        raise RuntimeError("row width is not a multiple of head_size")
+    q2 = query.view(n_tokens, query.shape[-1]) if query.is_contiguous() else None
+    k2 = key.view(n_tokens, key.shape[-1]) if key.is_contiguous() else None
+    q_stride = query.shape[-1] if q2 is not None else query.stride(-2)
+    k_stride = key.shape[-1] if k2 is not None else key.stride(-2)
+    if (q2 is None or k2 is None) and query.dim() != 2:
+        raise RuntimeError("strided query/key must be two-dimensional")
+    with torch.cuda.device(query.device):
+        stream = torch.cuda.current_stream(query.device).cuda_stream
+        _check(load().ca_rotary_embedding(positions.data_ptr(), query.data_ptr(), key.data_ptr(),
+                                          cos_sin_cache.data_ptr(), n_tokens, query.shape[-1] // head_size,
+                                          key.shape[-1] // head_size, head_size, cos_sin_cache.shape[1],
+                                          cos_sin_cache.shape[0], q_stride, k_stride, int(is_neox), stream))
+
+
 def max_chunks_for(memory_mb: int, chunk_size: int, n_heads: int, d_head: int, elem_bytes: int = 2) -> int:
     return load().ca_tree_max_chunks_for(memory_mb, chunk_size, n_heads, d_head, elem_bytes)
 
@@ -334,6 +373,11 @@ class KernelContext:
 
     def append_kv(self, k_ptr: int, v_ptr: int, n_seqs: int, stream: int = 0) -> None:
         _check(self._lib.ca_append_kv(self._h, k_ptr, v_ptr, n_seqs, stream))
+
+    def rope_append_kv(self, positions_ptr: int, q_ptr: int, k_ptr: int, v_ptr: int, cache_ptr: int,
+                       max_position: int, rot_dim: int, is_neox: bool, n_seqs: int, stream: int = 0) -> None:
+        _check(self._lib.ca_rope_append_kv(self._h, positions_ptr or None, q_ptr, k_ptr, v_ptr, cache_ptr,
+                                           max_position, rot_dim, int(is_neox), n_seqs, stream))
 
     def scatter_kv(self, k_ptr: int, v_ptr: int, n_tokens: int, tok_begin: int, slots: Sequence[int],
                    stream: int = 0) -> None:
@@ -477,6 +521,37 @@ class Attention:
         self.refresh_kernel_context()
         self.ctx.append_kv(k.data_ptr(), v.data_ptr(), len(tokens), self._stream())
         self.tree.append_token(tokens)  # reserve inside is a no-op now
+        self.ctx.delta_tokens = self.ctx.delta_tokens + 1
+        return n_new
+
+    def append_token_rotary(self, tokens: Sequence[int], q, k, v, cos_sin_cache, is_neox: bool = True,
+                            positions=None) -> int:
+        """append_token with the rotary embedding of the new rows folded in: q is rotated in
+        place, k is rotated on its way into the cache (k itself is left as it is), v is copied.
+        Without `positions` (int64 [n_seqs] on the device) a sequence's position is its length."""
+        import torch
+        if self.tree.n_seqs != len(tokens):
+            raise RuntimeError("num of seqs is not equal to num of tokens")
+        n = len(tokens)
+        k = self._check_kv(k, n, "k")
+        v = self._check_kv(v, n, "v")
+        if not q.is_contiguous() or q.dtype != torch.float16 or q.device != self.device or \
+                tuple(q.shape) != (n, self.n_heads, self.d_head):
+            raise RuntimeError(f"q must be contiguous fp16 [{n}, {self.n_heads}, {self.d_head}] on {self.device}")
+        if cos_sin_cache.dtype != torch.float16 or cos_sin_cache.device != self.device or \
+                cos_sin_cache.dim() != 2 or not cos_sin_cache.is_contiguous():
+            raise RuntimeError("cos_sin_cache must be contiguous fp16 [max_position, rot_dim] on the cache's device")
+        pos_ptr = 0
+        if positions is not None:
+            if positions.dtype != torch.int64 or positions.device != self.device or tuple(positions.shape) != (n,) \
+                    or not positions.is_contiguous():
+                raise RuntimeError(f"positions must be contiguous int64 [{n}] on {self.device}")
+            pos_ptr = positions.data_ptr()
+        n_new = self.reserve()
+        self.refresh_kernel_context()
+        self.ctx.rope_append_kv(pos_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_sin_cache.data_ptr(),
+                                cos_sin_cache.shape[0], cos_sin_cache.shape[1], is_neox, n, self._stream())
+        self.tree.append_token(tokens)
         self.ctx.delta_tokens = self.ctx.delta_tokens + 1
         return n_new
 

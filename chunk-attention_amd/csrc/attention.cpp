@@ -132,6 +132,45 @@ std::vector<Chunk*> Attention::append_token(const std::vector<int>& tokens, torc
     return fresh;
 }
 
+std::vector<Chunk*> Attention::append_token_rotary(const std::vector<int>& tokens, torch::Tensor q,
+                                                   torch::Tensor k, torch::Tensor v,
+                                                   torch::Tensor cos_sin_cache, bool is_neox,
+                                                   c10::optional<torch::Tensor> positions) {
+    if (tree_->tails().size() != tokens.size()) {
+        throw std::runtime_error("num of seqs is not equal to num of tokens");
+    }
+    const int n = static_cast<int>(tokens.size());
+    k = checked_kv(k, n, "k");
+    v = checked_kv(v, n, "v");
+    if (!q.is_contiguous() || q.scalar_type() != torch::kFloat16 || q.device() != t_options_.device() ||
+        q.dim() != 3 || q.size(0) != n || q.size(1) != n_heads_ || q.size(2) != d_head_) {
+        throw std::runtime_error("q must be contiguous float16 [n_seqs, n_heads, d_head] on the cache's device");
+    }
+    if (!cos_sin_cache.is_contiguous() || cos_sin_cache.scalar_type() != torch::kFloat16 ||
+        cos_sin_cache.device() != t_options_.device() || cos_sin_cache.dim() != 2) {
+        throw std::runtime_error("cos_sin_cache must be contiguous float16 [max_position, rot_dim] on the cache's device");
+    }
+    const int64_t* pos = nullptr;
+    if (positions.has_value() && positions->defined()) {
+        if (!positions->is_contiguous() || positions->scalar_type() != torch::kInt64 ||
+            positions->device() != t_options_.device() || positions->numel() != n) {
+            throw std::runtime_error("positions must be contiguous int64 [n_seqs] on the cache's device");
+        }
+        pos = positions->data_ptr<int64_t>();
+    }
+    std::vector<Chunk*> fresh = tree_->reserve();
+    refresh_kernel_context();
+    {
+        c10::DeviceGuard guard(t_options_.device());
+        check(ca_rope_append_kv(ctx_, pos, q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_sin_cache.data_ptr(),
+                                static_cast<int>(cos_sin_cache.size(0)), static_cast<int>(cos_sin_cache.size(1)),
+                                is_neox ? 1 : 0, n, stream()));
+    }
+    tree_->append_token_ids(tokens);
+    ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1);
+    return fresh;
+}
+
 torch::Tensor Attention::forward(torch::Tensor q, int partition) {
     if (!q.is_contiguous()) throw std::runtime_error("q is not contiguous");
     if (q.dim() != 3 || q.size(1) != n_heads_ || q.size(2) != d_head_) {
@@ -190,6 +229,36 @@ void Attention::print(Chunk* root, int level) {
     if (root == nullptr) root = tree_->root();
     std::cout << std::string(size_t(level) * 4, ' ') << root->to_string(true) << std::endl;
     for (Chunk* child : root->children) print(child, level + 1);
+}
+
+void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Tensor& key, int head_size,
+                      torch::Tensor& cos_sin_cache, bool is_neox) {
+    TORCH_CHECK(query.is_cuda() && key.is_cuda() && cos_sin_cache.is_cuda() && positions.is_cuda(),
+                "rotary_embedding: tensors must be on the GPU");
+    TORCH_CHECK(query.scalar_type() == torch::kFloat16 && key.scalar_type() == torch::kFloat16 &&
+                  cos_sin_cache.scalar_type() == torch::kFloat16,
+                "rotary_embedding: float16 only");
+    TORCH_CHECK(positions.scalar_type() == torch::kInt64 && positions.is_contiguous(),
+                "rotary_embedding: positions must be contiguous int64");
+    TORCH_CHECK(cos_sin_cache.dim() == 2 && cos_sin_cache.is_contiguous(), "rotary_embedding: cos_sin_cache must be [max_position, rot_dim]");
+    TORCH_CHECK(query.dim() >= 2 && key.dim() >= 2 && query.stride(-1) == 1 && key.stride(-1) == 1,
+                "rotary_embedding: rows must be contiguous");
+    const int64_t n_tokens = query.numel() / query.size(-1);
+    TORCH_CHECK(positions.numel() == n_tokens && key.numel() / key.size(-1) == n_tokens,
+                "rotary_embedding: positions, query and key disagree on the number of tokens");
+    TORCH_CHECK(query.size(-1) % head_size == 0 && key.size(-1) % head_size == 0,
+                "rotary_embedding: row width is not a multiple of head_size");
+    // as in the reference, tokens are query.stride(-2) elements apart (leading dims contiguous)
+    c10::DeviceGuard guard(query.device());
+    void* st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(query.device().index()).stream();
+    const int rc = ca_rotary_embedding(positions.data_ptr<int64_t>(), query.data_ptr(), key.data_ptr(),
+                                       cos_sin_cache.data_ptr(), n_tokens,
+                                       static_cast<int>(query.size(-1) / head_size),
+                                       static_cast<int>(key.size(-1) / head_size), head_size,
+                                       static_cast<int>(cos_sin_cache.size(1)),
+                                       static_cast<int>(cos_sin_cache.size(0)), query.stride(-2),
+                                       key.stride(-2), is_neox ? 1 : 0, st);
+    if (rc != 0) throw std::runtime_error(ca_last_error());
 }
 
 }  // namespace GPT

@@ -36,6 +36,15 @@ class Attention {
     // one token per sequence; k, v: [n_seqs, n_heads, d_head]
     std::vector<Chunk*> append_token(const std::vector<int>& tokens, torch::Tensor k,
                                      torch::Tensor v, bool fused = true);
+    // append_token with the rotary embedding of the new rows folded into the same launch
+    // (the reference's layer runs rotary_embedding, then append_token:
+    // src/chunk_attn/models/llama_hf/modeling_llama.py:62,91-95).  q [n_seqs, n_heads, d_head] is
+    // rotated in place; k is rotated on its way into the cache and itself left unchanged.
+    // positions: int64 [n_seqs] on the device, or an undefined tensor = each sequence's length.
+    std::vector<Chunk*> append_token_rotary(const std::vector<int>& tokens, torch::Tensor q,
+                                            torch::Tensor k, torch::Tensor v,
+                                            torch::Tensor cos_sin_cache, bool is_neox = true,
+                                            c10::optional<torch::Tensor> positions = c10::nullopt);
     void refresh_kernel_context(bool force = false);
     std::vector<Chunk*> reserve();
     void clear();
@@ -71,5 +80,10 @@ class Attention {
     ca_ctx* ctx_ = nullptr;
     uint64_t tables_version_ = 0;  // tree version the device tables were built from
 };
+
+// In-place rotary embedding of fp16 query/key rows: the operator the reference exports as
+// chunk_attn.ops.rotary_embedding (cpp/chunk_attn/pos_encoding_kernels.cu:94-139).
+void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Tensor& key, int head_size,
+                      torch::Tensor& cos_sin_cache, bool is_neox);
 
 }  // namespace GPT

@@ -144,7 +144,7 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
 
 int launch_rc(int rc, const char* what) {
     if (rc == 0) return CA_OK;
-    if (rc < 0) return fail(CA_ERR_INVALID, std::string(what) + ": unsupported chunk_size");
+    if (rc < 0) return fail(CA_ERR_INVALID, std::string(what) + ": unsupported shape");
     return fail_hip(static_cast<hipError_t>(rc), what);
 }
 
@@ -471,6 +471,74 @@ int ca_append_kv(ca_ctx* c, const void* k, const void* v, int n_seqs, void* stre
     return launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
                                        reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
                                        n_seqs, static_cast<hipStream_t>(stream)), "append launch");
+}
+
+int ca_rotary_embedding(const int64_t* positions, void* query, void* key, const void* cos_sin_cache,
+                        int64_t n_tokens, int n_heads, int n_kv_heads, int head_size, int rot_dim,
+                        int max_position, int64_t query_stride, int64_t key_stride, int is_neox,
+                        void* stream) {
+    if (n_tokens < 0 || n_heads < 0 || n_kv_heads < 0 || head_size <= 0 || max_position <= 0) {
+        return fail(CA_ERR_INVALID, "bad argument");
+    }
+    if (rot_dim <= 0 || rot_dim % 2 != 0 || rot_dim > head_size) {
+        return fail(CA_ERR_INVALID, "rot_dim must be even and within [2, head_size]");
+    }
+    if (n_tokens == 0 || n_heads + n_kv_heads == 0) return CA_OK;
+    if (!positions || !cos_sin_cache || (n_heads > 0 && !query) || (n_kv_heads > 0 && !key)) {
+        return fail(CA_ERR_INVALID, "null device pointer");
+    }
+    if (query_stride < int64_t(n_heads) * head_size || key_stride < int64_t(n_kv_heads) * head_size) {
+        return fail(CA_ERR_INVALID, "token stride smaller than a token's row");
+    }
+    ca::RotaryArgs r;
+    r.positions = positions;
+    r.query = query;
+    r.key = key;
+    r.cos_sin_cache = cos_sin_cache;
+    r.n_tokens = n_tokens;
+    r.n_heads = n_heads;
+    r.n_kv_heads = n_kv_heads;
+    r.head_size = head_size;
+    r.rot_dim = rot_dim;
+    r.max_position = max_position;
+    r.query_stride = query_stride;
+    r.key_stride = key_stride;
+    r.is_neox = is_neox != 0;
+    return launch_rc(ca::launch_rotary(r, static_cast<hipStream_t>(stream)), "rotary launch");
+}
+
+int ca_rope_append_kv(ca_ctx* c, const int64_t* positions, void* q, const void* k, const void* v,
+                      const void* cos_sin_cache, int max_position, int rot_dim, int is_neox,
+                      int n_seqs, void* stream) {
+    if (int rc = check_ready(c, k, n_seqs)) return rc;
+    if (n_seqs > 0 && (!v || !q || !cos_sin_cache)) return fail(CA_ERR_INVALID, "null device pointer");
+    if (max_position <= 0 || rot_dim <= 0 || rot_dim > c->d || rot_dim % (is_neox ? 16 : 8) != 0) {
+        return fail(CA_ERR_INVALID, "rot_dim must be a multiple of 16 (NeoX) or 8 (GPT-J) within d_head, max_position positive");
+    }
+    if (c->d % 8 != 0 || 64 % (c->d / 8) != 0) {
+        return fail(CA_ERR_INVALID, "fused rotary append needs d_head in {8, 16, 32, 64, 128, 256, 512}");
+    }
+    for (int s = 0; s < n_seqs; s++) {
+        if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
+            return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
+        }
+        if (!positions && c->plan.seq_len[s] + c->delta_tokens >= max_position) {
+            return fail(CA_ERR_INVALID, "sequence " + std::to_string(s) + " is longer than the cos/sin cache");
+        }
+    }
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    ca::RotaryArgs r;
+    r.positions = positions;
+    r.query = q;
+    r.cos_sin_cache = cos_sin_cache;
+    r.rot_dim = rot_dim;
+    r.max_position = max_position;
+    r.is_neox = is_neox != 0;
+    return launch_rc(ca::launch_rope_append(a, r, k, v,
+                                            reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len),
+                                            reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
+                                            reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
+                                            n_seqs, static_cast<hipStream_t>(stream)), "rotary append launch");
 }
 
 int ca_scatter_kv(ca_ctx* c, const void* k, const void* v, int n_tokens, int tok_begin,

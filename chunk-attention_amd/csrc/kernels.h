@@ -46,4 +46,24 @@ int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,
                    const int32_t* slots, int n_slots, hipStream_t st);
 
+// Rotary position embedding (fp16).  cos_sin_cache is [max_position, rot_dim]: rot_dim/2 cosines
+// then rot_dim/2 sines per position; positions outside the cache are clamped into it.
+struct RotaryArgs {
+    const int64_t* positions = nullptr;  // device, one per token; may be null for launch_rope_append
+    void* query = nullptr;               // rotated in place
+    void* key = nullptr;                 // rotated in place (launch_rotary only; may be null with n_kv_heads 0)
+    const void* cos_sin_cache = nullptr;
+    int64_t n_tokens = 0;
+    int n_heads = 0, n_kv_heads = 0, head_size = 0, rot_dim = 0, max_position = 0;
+    int64_t query_stride = 0, key_stride = 0;  // elements between consecutive tokens
+    bool is_neox = true;
+};
+int launch_rotary(const RotaryArgs& r, hipStream_t st);
+// One launch for a decode step's new rows: r.query ([n_seqs, H, d]) is rotated in place, k is
+// rotated on its way into the free row of each sequence's last chunk, v is copied beside it.
+// The position of sequence s is r.positions[s] or, when that is null, seq_len[s] + delta_tokens.
+int launch_rope_append(const LaunchArgs& a, const RotaryArgs& r, const void* k, const void* v,
+                       const int32_t* seq_len, const int32_t* tail_slot, const int32_t* tail_fill,
+                       int n_seqs, hipStream_t st);
+
 }  // namespace ca

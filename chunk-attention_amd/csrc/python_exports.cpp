@@ -45,6 +45,9 @@ PYBIND11_MODULE(chunk_attn_c, m) {
       .def("add_seq_async", &Attention::add_seq_async, py::arg("tokens"), py::arg("k"), py::arg("v"))
       .def("append_token", &Attention::append_token, py::arg("tokens"), py::arg("k"), py::arg("v"),
            py::arg("fused") = true, py::return_value_policy::reference)
+      .def("append_token_rotary", &Attention::append_token_rotary, py::arg("tokens"), py::arg("q"), py::arg("k"),
+           py::arg("v"), py::arg("cos_sin_cache"), py::arg("is_neox") = true, py::arg("positions") = py::none(),
+           py::return_value_policy::reference)
       .def("refresh_kernel_context", &Attention::refresh_kernel_context, py::arg("force") = false)
       .def("reserve", &Attention::reserve, py::return_value_policy::reference)
       .def("duplicate", &Attention::duplicate, py::arg("seq_idx"), py::arg("copies"))
@@ -65,4 +68,11 @@ PYBIND11_MODULE(chunk_attn_c, m) {
            py::return_value_policy::reference)
       .def("key", &Attention::key, py::arg("chunk"))
       .def("value", &Attention::value, py::arg("chunk"));
+
+    // the reference's chunk_attn.ops module (cpp/chunk_attn/python_exports_ops.cpp:11-19), the part the
+    // decode path's caller uses
+    py::module ops = m.def_submodule("ops", "operators used around the attention call");
+    ops.def("rotary_embedding", &GPT::rotary_embedding, py::arg("positions"), py::arg("query"), py::arg("key"),
+            py::arg("head_size"), py::arg("cos_sin_cache"), py::arg("is_neox"),
+            "Apply GPT-NeoX or GPT-J style rotary embedding to query and key");
 }

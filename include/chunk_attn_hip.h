@@ -93,6 +93,32 @@ int ca_attn_seqs_first(ca_ctx* ctx, const void* q, void* out, int n_seqs, void* 
  * per sequence at position seq_len + delta_tokens.  Does not change delta_tokens. */
 int ca_append_kv(ca_ctx* ctx, const void* k, const void* v, int n_seqs, void* stream);
 
+/* Replaces rotary_embedding(positions, query, key, head_size, cos_sin_cache, is_neox)
+ * (cpp/chunk_attn/pos_encoding_kernels.cu:94-139, bound as chunk_attn.ops.rotary_embedding in
+ * cpp/chunk_attn/python_exports_ops.cpp:13): rotates query and key rows in place, fp16 only.
+ * positions: n_tokens int64 on the device.  query: n_tokens rows of n_heads*head_size halves,
+ * query_stride elements apart; key likewise with n_kv_heads (key may be NULL with
+ * n_kv_heads 0).  cos_sin_cache: [max_position, rot_dim] halves, rot_dim/2 cosines then
+ * rot_dim/2 sines per position.  is_neox != 0 pairs element r with r + rot_dim/2 (GPT-NeoX),
+ * else 2r with 2r+1 (GPT-J).  Products are formed in fp32 and rounded to fp16 once; positions
+ * outside [0, max_position) are clamped into the cache instead of read out of bounds. */
+int ca_rotary_embedding(const int64_t* positions_dev, void* query, void* key,
+                        const void* cos_sin_cache, int64_t n_tokens, int n_heads,
+                        int n_kv_heads, int head_size, int rot_dim, int max_position,
+                        int64_t query_stride, int64_t key_stride, int is_neox, void* stream);
+
+/* The decode step of the reference's attention layer
+ * (src/chunk_attn/models/llama_hf/modeling_llama.py:62,91-95: rotary_embedding on the new
+ * query/key rows, then append_token -> append_kv) as one launch: q [n_seqs, n_heads, d_head]
+ * is rotated in place, k is rotated on its way into the free row of each sequence's last
+ * chunk (k itself is left untouched), v is copied beside it.  positions_dev may be NULL: the
+ * position of a sequence is then its current length, seq_len + delta_tokens, checked against
+ * max_position on the host.  Same preconditions and delta_tokens behaviour as ca_append_kv;
+ * rot_dim must be a multiple of 16 (NeoX) or 8 (GPT-J) and at most d_head. */
+int ca_rope_append_kv(ca_ctx* ctx, const int64_t* positions_dev, void* q, const void* k,
+                      const void* v, const void* cos_sin_cache, int max_position, int rot_dim,
+                      int is_neox, int n_seqs, void* stream);
+
 /* Copy-in of an inserted sequence's K/V (what the reference does with two tensor slice
  * assignments per chunk, cpp/chunk_attn/chunk.cpp:63-72): token rows
  * [tok_begin, tok_begin + n_slots*chunk_size) clipped to n_tokens go to the listed chunks,

@@ -191,3 +191,60 @@ def test_errors_and_defaults(mod):
             attn.add_seq(tokens=[100 + i] * 64, k=torch.ones((64, 2, 128), dtype=torch.float16, device="cuda"),
                          v=torch.ones((64, 2, 128), dtype=torch.float16, device="cuda"))
     attn.print()
+
+
+def test_rotary_ops_and_fused_append_match_the_c_abi_binding(mod):
+    """chunk_attn.ops.rotary_embedding (reference python_exports_ops.cpp:13) and
+    Attention.append_token_rotary go through the same C-ABI entry points as the ctypes binding:
+    identical results, and the fused step equals rotary followed by append_token."""
+    from chunk_attn import capi
+    from oracle.rotary import cos_sin_cache, rotary_embedding
+    rng = np.random.default_rng(21)
+    H, d, c, n = 2, 128, 32, 3
+    cache_np = cos_sin_cache(d, 256)
+    cache = torch.from_numpy(cache_np).cuda()
+    pos_np = np.array([5, 0, 77], dtype=np.int64)
+    q_np = rng.standard_normal((n, H * d)).astype(np.float16)
+    k_np = rng.standard_normal((n, H * d)).astype(np.float16)
+    q, k, pos = torch.from_numpy(q_np).cuda(), torch.from_numpy(k_np).cuda(), torch.from_numpy(pos_np).cuda()
+    mod.ops.rotary_embedding(pos, q, k, d, cache, True)
+    q2, k2 = torch.from_numpy(q_np).cuda(), torch.from_numpy(k_np).cuda()
+    capi.rotary_embedding(pos, q2, k2, d, cache, True)
+    assert torch.equal(q, q2) and torch.equal(k, k2)
+    wq, wk = rotary_embedding(pos_np, q_np, k_np, d, cache_np, True)
+    np.testing.assert_allclose(q.float().cpu().numpy(), wq.astype(np.float32), atol=2e-3, rtol=1e-2)
+    np.testing.assert_allclose(k.float().cpu().numpy(), wk.astype(np.float32), atol=2e-3, rtol=1e-2)
+
+    def cache_with_two_seqs():
+        a = mod.Attention(n_heads=H, d_head=d, chunk_size=c, memory_mb=4, dtype=torch.float16,
+                          device=torch.device("cuda"))
+        g = torch.Generator().manual_seed(3)
+        for s, T in enumerate((40, 45)):
+            toks = list(range(32)) + [1000 * (s + 1) + i for i in range(T - 32)]
+            kk = torch.randn((T, H, d), generator=g).half()
+            vv = torch.randn((T, H, d), generator=g).half()
+            if s:
+                kk[:32], vv[:32] = first[0][:32], first[1][:32]
+            else:
+                first = (kk, vv)
+            assert a.add_seq(tokens=toks, k=kk.cuda(), v=vv.cuda()) == s
+        return a
+
+    fused, plain = cache_with_two_seqs(), cache_with_two_seqs()
+    for step in range(30):      # sequence 0 crosses into a new chunk at step 24
+        qn = torch.randn((2, H, d)).half().cuda()
+        kn = torch.randn((2, H, d)).half().cuda()
+        vn = torch.randn((2, H, d)).half().cuda()
+        lens = torch.tensor([40 + step, 45 + step], dtype=torch.int64, device="cuda")
+        qf, qp, kp = qn.clone(), qn.clone(), kn.clone()
+        fresh = fused.append_token_rotary(tokens=[step, step], q=qf, k=kn, v=vn, cos_sin_cache=cache)
+        mod.ops.rotary_embedding(lens, qp.view(2, H * d), kp.view(2, H * d), d, cache, True)
+        fresh_p = plain.append_token(tokens=[step, step], k=kp, v=vn)
+        assert len(fresh) == len(fresh_p)
+        # same fp32 arithmetic in both kernels; the final rounding to fp16 may differ by one place
+        assert ((qf.float() - qp.float()).abs() <= 2.0 ** -10 * qf.float().abs() + 2.0 ** -24).all()
+        np.testing.assert_allclose(fused.forward(qf).float().cpu().numpy(), plain.forward(qp).float().cpu().numpy(),
+                                   atol=2e-3, rtol=1e-2)
+    with pytest.raises(RuntimeError, match="positions"):
+        fused.append_token_rotary(tokens=[1, 2], q=qf, k=kn, v=vn, cos_sin_cache=cache,
+                                  positions=torch.zeros(3, dtype=torch.int64, device="cuda"))
