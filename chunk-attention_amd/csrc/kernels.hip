@@ -87,6 +87,17 @@ __device__ __forceinline__ uint4 nt_load16(const uint4* p) {
     return make_uint4(v[0], v[1], v[2], v[3]);
 }
 
+// LDS transpose read (gfx950): within each group of 16 lanes, lane L supplies the address of four
+// consecutive halves; with lane L pointing at row L/4, columns 4*(L%4).. of a 4 x 16 patch, lane i
+// receives column i of the patch (rows 0..3).  That is the V^T operand of the matrix cores,
+// lane (i = dim, g = token group), straight from a row-major V tile.
+__device__ __forceinline__ h4 lds_read_tr(const half_t* p) {
+    // p points into LDS: the cast narrows the generic pointer to the LDS address space
+    typedef short s4v __attribute__((ext_vector_type(4)));
+    const s4v raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4v __attribute__((address_space(3)))*)p);
+    return __builtin_bit_cast(h4, raw);
+}
+
 __device__ __forceinline__ float dot8(const h8& a, const h8& b, float acc) {
     acc = __builtin_amdgcn_fdot2(h2{ a[0], a[1] }, h2{ b[0], b[1] }, acc, false);
     acc = __builtin_amdgcn_fdot2(h2{ a[2], a[3] }, h2{ b[2], b[3] }, acc, false);
@@ -152,6 +163,25 @@ __device__ __forceinline__ float reduce_rows16(float (&v)[NV], int j) {
 __device__ __forceinline__ int item_slot(const WorkItem* __restrict__ gi, int slot_first,
                                          const int32_t* __restrict__ slots, int k) {
     return k < kInlineSlots ? gi->inl[k] : slots[slot_first + k];
+}
+
+// Every wave fetches the slot ids of its item's first 64 chunks with one load, chunk k into lane
+// k, when it starts: looking a slot up in memory right before the chunk's K/V loads would put
+// a dependent round trip in front of every tile.  chunk_slot reads it back from the register.
+__device__ __forceinline__ int preload_slots(const WorkItem* __restrict__ gi, int slot_first, int n_chunks,
+                                             const int32_t* __restrict__ slots, int lane) {
+    // the item's inline slots do not wait for the item's header: they arrive with it
+    int v = 0;
+    if (lane < kInlineSlots) {
+        v = gi->inl[lane];
+    } else if (lane < n_chunks) {
+        v = slots[slot_first + lane];
+    }
+    return v;
+}
+// k must be the same in every lane of the wave.
+__device__ __forceinline__ int chunk_slot(int slotv, int slot_first, const int32_t* __restrict__ slots, int k) {
+    return k < 64 ? __builtin_amdgcn_readlane(slotv, k) : slots[slot_first + k];
 }
 
 // Everything a workgroup needs besides its work item.
@@ -221,8 +251,9 @@ __device__ __forceinline__ void merge_rows(const float* __restrict__ part, int p
 }
 
 // LDS of one workgroup, shared by the two paths.
-constexpr int VPITCH = D + 4;  // halves per LDS row of a V block: 264 B keeps the four token
-                               // groups on disjoint banks for 2-byte column reads
+constexpr int VPITCH = D + 16;  // halves per LDS row of a V block: 288 B puts the 32-byte pieces of
+                                // four consecutive token rows into four different bank groups,
+                                // and rows stay 16-byte aligned for whole-vector writes
 constexpr int OPITCH = D + 4;  // floats per row of the cross-wave accumulation buffer
 constexpr int MB = 2;          // 16-row blocks per shared item
 constexpr int MROWS = 16 * MB;
@@ -272,7 +303,9 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     constexpr int NSUB = C / SUB;
 
     const int tid = threadIdx.x;
-    const int w = tid >> 6, l = tid & 63, g = l >> 4, j = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
+    const int l = tid & 63, g = l >> 4, j = l & 15;
+    const int slotv = preload_slots(gi, it.slot_first, it.n_chunks, slots, l);
     const int seq = it.seq_begin;
     const int len = it.len0 + A.delta_tokens;
 
@@ -340,7 +373,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
         int valid = len - (it.pos0 + t) * C;
         if (valid <= 0) break;  // chunks are in path order: everything after is empty too
         valid = valid < C ? valid : C;
-        const int slot = item_slot(gi, it.slot_first, slots, t);
+        const int slot = chunk_slot(slotv, it.slot_first, slots, t);
         const size_t base = (size_t(slot) * H + h) * size_t(C) * D;
 #pragma unroll
         for (int sub = 0; sub < NSUB; sub++) {
@@ -500,7 +533,9 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
     const int tid = threadIdx.x;
-    const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
+    const int l = tid & 63, g = l >> 4, i = l & 15;
+    const int slotv = preload_slots(gi, it.slot_first, it.n_chunks, slots, l);
     const int len = it.len0 + A.delta_tokens;
     const bool two = it.n_rows > 16;  // second 16-row block in use (uniform)
     if (tid < it.n_rows) sm.row[tid] = A.part_ptr[it.seq_begin + tid] + it.part_row;
@@ -532,7 +567,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     // valid tokens of block tb (<= 0: past the end of the sequence), and its element offset
     auto block_valid = [&](int tb) { return len - (it.pos0 + tb / BPC) * C - (tb % BPC) * 16; };
     auto block_base = [&](int tb) {
-        return ((size_t(item_slot(gi, it.slot_first, slots, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
+        return ((size_t(chunk_slot(slotv, it.slot_first, slots, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
     };
     h8 kreg[4], knext[4];
     uint4 vraw[4], vnext[4];
@@ -560,9 +595,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
         for (int r = 0; r < 4; r++) {
             uint4 t = vraw[r];
             if (4 * r + g >= valid) t = make_uint4(0, 0, 0, 0);
-            uint2* dst = reinterpret_cast<uint2*>(&sm.v[w][(4 * r + g) * VPITCH + 8 * i]);
-            dst[0] = make_uint2(t.x, t.y);
-            dst[1] = make_uint2(t.z, t.w);
+            *reinterpret_cast<uint4*>(&sm.v[w][(4 * r + g) * VPITCH + 8 * i]) = t;
         }
 
         h4 pb[MB];
@@ -605,8 +638,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
         // O^T += V^T . P^T : A = V^T (row = dim 16*db + i, k = tokens 4g..4g+3)
 #pragma unroll
         for (int db = 0; db < 8; db++) {
-            const half_t* col = &sm.v[w][(4 * g) * VPITCH + 16 * db + i];
-            const h4 a = h4{ col[0], col[VPITCH], col[2 * VPITCH], col[3 * VPITCH] };
+            const h4 a = lds_read_tr(&sm.v[w][(4 * g + (i >> 2)) * VPITCH + 16 * db + 4 * (i & 3)]);
             oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[0], oacc[0][db], 0, 0, 0);
             if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1], oacc[1][db], 0, 0, 0);
         }
@@ -718,11 +750,12 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
     const int tid = threadIdx.x;
-    const int w = tid >> 6, l = tid & 63, g = l >> 4, i = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
+    const int l = tid & 63, g = l >> 4, i = l & 15;
+    const int slotv = preload_slots(gi, it.slot_first, it.n_chunks, slots, l);
     const int len = it.len0 + A.delta_tokens;
     const int row_base = 32 * w;                    // first item row of this wave
     const bool active = row_base < it.n_rows;       // wave has sequences (uniform per wave)
-    const bool two = row_base + 16 < it.n_rows;
 
     h8 qreg[MB][4];
 #pragma unroll
@@ -754,10 +787,12 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
         for (int r = 0; r < 4; r++) {
             const int p = tid + 256 * r;
             const int tok = 64 * t + (p >> 4);  // token of the segment
-            const int ck = tok / C;
+            // the 16 token rows the workgroup stages in step r lie in one chunk (chunk sizes are
+            // multiples of 16): the chunk index is uniform
+            const int ck = (64 * t + 16 * r) / C;
             const int valid = len - (it.pos0 + ck) * C - (tok % C);  // > 0: token exists
             if (tok < total_tokens && valid > 0) {
-                const size_t off = ((size_t(item_slot(gi, it.slot_first, slots, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
+                const size_t off = ((size_t(chunk_slot(slotv, it.slot_first, slots, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
                 kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
                 vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
             } else {
@@ -783,9 +818,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
         for (int r = 0; r < 4; r++) {
             const int p = tid + 256 * r;
             *reinterpret_cast<uint4*>(&sm.k[(p >> 4) * KPITCH + 8 * (p & 15)]) = kst[r];
-            uint2* dv = reinterpret_cast<uint2*>(&sm.v[(p >> 4) * VPITCH + 8 * (p & 15)]);
-            dv[0] = make_uint2(vst[r].x, vst[r].y);
-            dv[1] = make_uint2(vst[r].z, vst[r].w);
+            *reinterpret_cast<uint4*>(&sm.v[(p >> 4) * VPITCH + 8 * (p & 15)]) = vst[r];
         }
         __syncthreads();
         if (t + 1 < n_tiles) fetch_tile(t + 1);
@@ -802,12 +835,12 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
             }
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) {
+                // rows past the item's last sequence carry zero queries: computed, never stored
+                // (no branch in this loop, so that LDS reads and matrix ops can be pipelined)
                 f4 acc = f4{ 0.f, 0.f, 0.f, 0.f };
-                if (mb == 0 || two) {
 #pragma unroll
-                    for (int ks = 0; ks < 4; ks++) {
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[ks], qreg[mb][ks], acc, 0, 0, 0);
-                    }
+                for (int ks = 0; ks < 4; ks++) {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[ks], qreg[mb][ks], acc, 0, 0, 0);
                 }
                 sc[mb][tb] = acc;
             }
@@ -845,15 +878,31 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
 #pragma unroll
             for (int db = 0; db < 8; db++) oacc[mb][db] *= alpha;
         }
-        // O^T += V^T . P^T
+        // O^T += V^T . P^T with k = 32 tokens per instruction: k-slot (g, e) stands for token
+        // 4g + e of 16-token block 2*tp (e < 4) or 2*tp + 1 (e >= 4) in both operands, which is
+        // where the S^T result layout already holds the probabilities
 #pragma unroll
-        for (int db = 0; db < 8; db++) {
+        for (int tp = 0; tp < 2; tp++) {
+            h8 pp[MB];
 #pragma unroll
-            for (int tb = 0; tb < 4; tb++) {
-                const half_t* col = &sm.v[(16 * tb + 4 * g) * VPITCH + 16 * db + i];
-                const h4 a = h4{ col[0], col[VPITCH], col[2 * VPITCH], col[3 * VPITCH] };
-                oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[0][tb], oacc[0][db], 0, 0, 0);
-                if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1][tb], oacc[1][db], 0, 0, 0);
+            for (int mb = 0; mb < MB; mb++) {
+                const h4 lo = pb[mb][2 * tp], hi = pb[mb][2 * tp + 1];
+                pp[mb] = h8{ lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+            }
+            // all eight V^T operands of this token pair are requested before the first matrix
+            // op waits for one: the reads' latencies overlap instead of adding up
+            h8 a[8];
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                const half_t* p0 = &sm.v[(32 * tp + 4 * g + (i >> 2)) * VPITCH + 16 * db + 4 * (i & 3)];
+                const h4 lo = lds_read_tr(p0), hi = lds_read_tr(p0 + 16 * VPITCH);
+                a[db] = h8{ lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[0], oacc[0][db], 0, 0, 0);
+                oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[1], oacc[1][db], 0, 0, 0);
             }
         }
     }
