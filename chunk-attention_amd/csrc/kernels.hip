@@ -158,16 +158,11 @@ __device__ __forceinline__ float reduce_rows16(float (&v)[NV], int j) {
 // Lane l = 16*g + j reads, for load i, the 16 bytes at offset 1024*i + 16*l of a sub-tile:
 // row 4*i + g, dims 8*j..8*j+7, so every load instruction covers 1 KiB of contiguous memory.
 // ---------------------------------------------------------------------------------------
-// Slot of the k-th chunk of an item: the first ones come with the item, the rest from the list.
-// (`gi` is the item in global memory: indexing a register copy dynamically would spill it.)
-__device__ __forceinline__ int item_slot(const WorkItem* __restrict__ gi, int slot_first,
-                                         const int32_t* __restrict__ slots, int k) {
-    return k < kInlineSlots ? gi->inl[k] : slots[slot_first + k];
-}
-
-// Every wave fetches the slot ids of its item's first 64 chunks with one load, chunk k into lane
-// k, when it starts: looking a slot up in memory right before the chunk's K/V loads would put
-// a dependent round trip in front of every tile.  chunk_slot reads it back from the register.
+// Every wave fetches the slot ids of its item's chunks (at most 64: kMaxItemChunks) with one
+// load, chunk k into lane k, when it starts.  Looking a slot up in memory right before the
+// chunk's K/V loads would put a dependent round trip in front of every tile, and waiting for
+// that load (the counter of outstanding loads is in-order) would also wait for every K/V load
+// issued before it.  chunk_slot reads the id back from the register.
 __device__ __forceinline__ int preload_slots(const WorkItem* __restrict__ gi, int slot_first, int n_chunks,
                                              const int32_t* __restrict__ slots, int lane) {
     // the item's inline slots do not wait for the item's header: they arrive with it
@@ -179,10 +174,8 @@ __device__ __forceinline__ int preload_slots(const WorkItem* __restrict__ gi, in
     }
     return v;
 }
-// k must be the same in every lane of the wave.
-__device__ __forceinline__ int chunk_slot(int slotv, int slot_first, const int32_t* __restrict__ slots, int k) {
-    return k < 64 ? __builtin_amdgcn_readlane(slotv, k) : slots[slot_first + k];
-}
+// k < 64, the same in every lane of the wave.
+__device__ __forceinline__ int chunk_slot(int slotv, int k) { return __builtin_amdgcn_readlane(slotv, k); }
 
 // Everything a workgroup needs besides its work item.
 struct DecodeArgs {
@@ -373,7 +366,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
         int valid = len - (it.pos0 + t) * C;
         if (valid <= 0) break;  // chunks are in path order: everything after is empty too
         valid = valid < C ? valid : C;
-        const int slot = chunk_slot(slotv, it.slot_first, slots, t);
+        const int slot = chunk_slot(slotv, t);
         const size_t base = (size_t(slot) * H + h) * size_t(C) * D;
 #pragma unroll
         for (int sub = 0; sub < NSUB; sub++) {
@@ -567,7 +560,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     // valid tokens of block tb (<= 0: past the end of the sequence), and its element offset
     auto block_valid = [&](int tb) { return len - (it.pos0 + tb / BPC) * C - (tb % BPC) * 16; };
     auto block_base = [&](int tb) {
-        return ((size_t(chunk_slot(slotv, it.slot_first, slots, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
+        return ((size_t(chunk_slot(slotv, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
     };
     h8 kreg[4], knext[4];
     uint4 vraw[4], vnext[4];
@@ -610,22 +603,25 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
             for (int ks = 0; ks < 4; ks++) {
                 s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[ks], qreg[mb][ks], s, 0, 0, 0);
             }
-            float mx = NEG_INF;
+            // raw-score maximum: the scale is positive and rides in the exponent's multiply-add.
+            // Masking is a select, not a branch: no branch may sit between a matrix op and the
+            // first use of its result (the compiler's wait states for that hazard do not reach
+            // across a taken branch).
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                s[r] = (4 * g + r < valid) ? s[r] * scale_log2 : NEG_INF;
-                mx = fmaxf(mx, s[r]);
+                if (4 * g + r >= valid) s[r] = NEG_INF;
             }
+            float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
             mx = fmaxf(mx, shfl_xor(mx, 16));
             mx = fmaxf(mx, shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run[mb], mx);
+            const float m_new = fmaxf(m_run[mb], mx * scale_log2);  // valid >= 1: mx is finite
             const float alpha = fast_exp2(m_run[mb] - m_new);
             m_run[mb] = m_new;
             float psum = 0.f;
             float p[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                p[r] = fast_exp2(s[r] - m_new);
+                p[r] = fast_exp2(__builtin_fmaf(s[r], scale_log2, -m_new));
                 psum += p[r];
             }
             l_lane[mb] = l_lane[mb] * alpha + psum;
@@ -792,7 +788,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
             const int ck = (64 * t + 16 * r) / C;
             const int valid = len - (it.pos0 + ck) * C - (tok % C);  // > 0: token exists
             if (tok < total_tokens && valid > 0) {
-                const size_t off = ((size_t(chunk_slot(slotv, it.slot_first, slots, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
+                const size_t off = ((size_t(chunk_slot(slotv, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
                 kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
                 vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
             } else {
@@ -845,6 +841,21 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
                 sc[mb][tb] = acc;
             }
         }
+        // online softmax on the raw scores: the row maximum is taken before scaling (the scale
+        // is positive) and the scale rides in the exponent's multiply-add.  Tokens past the end
+        // of the sequence are masked with selects, never with a branch: no branch may sit
+        // between a matrix op and the first use of its result (the wait states the compiler
+        // inserts for that hazard do not reach across a taken branch).
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (16 * tb + 4 * g + r >= valid) sc[mb][tb][r] = NEG_INF;
+                }
+            }
+        }
         h4 pb[MB][4];
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
@@ -852,15 +863,11 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
 #pragma unroll
             for (int tb = 0; tb < 4; tb++) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float v = (16 * tb + 4 * g + r < valid) ? sc[mb][tb][r] * scale_log2 : NEG_INF;
-                    sc[mb][tb][r] = v;
-                    mx = fmaxf(mx, v);
-                }
+                for (int r = 0; r < 4; r++) mx = fmaxf(mx, sc[mb][tb][r]);
             }
             mx = fmaxf(mx, shfl_xor(mx, 16));
             mx = fmaxf(mx, shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run[mb], mx);
+            const float m_new = fmaxf(m_run[mb], mx * scale_log2);  // valid >= 1: mx is finite
             const float alpha = fast_exp2(m_run[mb] - m_new);
             m_run[mb] = m_new;
             float psum = 0.f;
@@ -869,7 +876,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
                 float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    p[r] = fast_exp2(sc[mb][tb][r] - m_new);
+                    p[r] = fast_exp2(__builtin_fmaf(sc[mb][tb][r], scale_log2, -m_new));
                     psum += p[r];
                 }
                 pb[mb][tb] = h4{ half_t(p[0]), half_t(p[1]), half_t(p[2]), half_t(p[3]) };

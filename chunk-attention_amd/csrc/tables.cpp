@@ -114,7 +114,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     }
     const double step_us = double(all_tokens) * 4.0 * std::max(params.n_heads, 1) * 128.0 / 6.4e6;
     auto seg_chunks_for = [&](int n_covered) {
-        if (params.shared_seg_chunks > 0) return params.shared_seg_chunks;
+        if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
         const bool wide = n_covered >= kWideMin;
         const double tiles = wide ? 0.5 * step_us / 4.0 : 0.4 * step_us / 2.0;
         const int n_tiles = std::clamp(static_cast<int>(tiles), 4, 32);  // 64-token tiles
@@ -126,7 +126,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         const ChunkRow& r0 = rows[run.first_row];
         const int n = r0.seq_end - r0.seq_begin;
         const int seg = seg_chunks_for(n);
-        const int n_segs = std::max(1, (run.count + seg / 2) / seg);  // nearest, not ceiling
+        // nearest, not ceiling; but never more chunks in a segment than an item may hold
+        const int n_segs = std::max({ 1, (run.count + seg / 2) / seg, ceil_div(run.count, kMaxItemChunks) });
         for (int g = 0; g < n_segs; g++) {
             // spread chunks evenly over the segments of a run
             const int c0 = int(int64_t(run.count) * g / n_segs);
@@ -185,6 +186,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             stream_chunks /= 2;
         }
     }
+    stream_chunks = std::min(stream_chunks, kMaxItemChunks - 1);  // an item may take one chunk more
     for (int s = 0; s < n_seqs; s++) {
         const auto& own = own_rows[s];
         if (own.empty()) continue;
@@ -233,6 +235,15 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         p.max_parts_per_seq = std::max(p.max_parts_per_seq, n_parts[s]);
     }
     p.n_part_rows = p.part_ptr[n_seqs];
+
+    // what the kernels assume about every item
+    for (const auto* list : { &p.shared_items, &p.stream_items }) {
+        for (const WorkItem& it : *list) {
+            if (it.n_chunks < 1 || it.n_chunks > kMaxItemChunks) {
+                throw std::logic_error("tables: work item with an unsupported number of chunks");
+            }
+        }
+    }
 }
 
 }  // namespace ca

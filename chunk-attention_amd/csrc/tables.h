@@ -40,12 +40,15 @@ void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_si
 // and the first chunk slots sit in the item itself so that a workgroup can issue its first K/V
 // loads after a single memory round trip.
 constexpr int kInlineSlots = 8;
+// No item holds more chunks than a wavefront has lanes: every wave keeps its item's slot ids in
+// one register, chunk k in lane k.
+constexpr int kMaxItemChunks = 64;
 struct WorkItem {
     int32_t seq_begin;   // first sequence (row of q) this item attends for
     int32_t n_rows;      // sequences covered (1 for stream items, <= kMaxRows for shared,
                          // <= kWideRows for wide shared items)
     int32_t slot_first;  // index into Plan::slots of the item's first chunk
-    int32_t n_chunks;    // consecutive entries of Plan::slots
+    int32_t n_chunks;    // consecutive entries of Plan::slots, <= kMaxItemChunks
     int32_t part_row;    // which of its sequence's partial rows the item writes: row
                          // part_ptr[seq] + part_row (for every covered sequence of a shared
                          // item); -1: the item writes the final output directly
