@@ -271,3 +271,27 @@ def test_repeated_forwards_are_bit_identical(c):
             junk = torch.randn(4096, device=dev())     # moves the allocator's free blocks around
             assert torch.equal(attn.forward(to_dev(q), partition), first)
             del junk
+
+
+@pytest.mark.parametrize("c", [32, 64])
+def test_long_paths_split_into_items_of_at_most_64_chunks(c):
+    """Sequences far longer than 64 chunks, with plan sizes asked for beyond what an item may
+    hold: the work list is capped and every partition still matches the oracle."""
+    rng = np.random.default_rng(50)
+    H, B = 2, 3
+    P, U = 70 * c, 75 * c + 7          # 70 shared chunks, 76 private chunks per sequence
+    sk, sv = rand16(rng, P, H, 128), rand16(rng, P, H, 128)
+    attn = make_attention(H, c, 70 + B * 78)
+    for s in range(B):
+        k, v = rand16(rng, P + U, H, 128), rand16(rng, P + U, H, 128)
+        k[:P], v[:P] = sk, sv
+        assert attn.add_seq(list(range(P)) + [10_000_000 * (s + 1) + i for i in range(U)], to_dev(k), to_dev(v)) == s
+    q = rand16(rng, B, H, 128)
+    want = oracle_output(attn, q, exact=True)
+    for seg, strm in ((0, 0), (400, 400)):
+        attn.ctx.set_plan(seg, strm)
+        for partition in (0, 1, 2):
+            assert_close(attn.forward(to_dev(q), partition), want)
+            tables = capi.build_tables(attn.get_chunks(), B, c, 1, partition, seg, strm, n_heads=H)
+            for items in (tables["plan"]["shared_items"], tables["plan"]["stream_items"]):
+                assert len(items) == 0 or items[:, 3].max() <= 64

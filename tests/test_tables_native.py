@@ -146,3 +146,23 @@ def test_bad_rows_rejected():
         capi.build_tables(rows, 2, 2)          # range exceeds n_seqs
     with pytest.raises(capi.ChunkAttnError):
         capi.build_tables(rows, 3, 2, partition=5)
+
+
+@pytest.mark.parametrize("partition", [0, 1, 2])
+@pytest.mark.parametrize("seg,strm", [(0, 0), (500, 500), (64, 63), (65, 64)])
+def test_items_never_hold_more_than_64_chunks(partition, seg, strm):
+    """The kernels keep an item's slot ids in one register per wave (64 lanes): whatever segment
+    or stream sizes are asked for, no work item may exceed 64 chunks, and all chunks are still
+    covered exactly once."""
+    c = 2
+    t = PrefixTree(c, 4096)
+    shared = list(range(2 * 150))                 # 150 shared chunks on one path
+    for s in range(5):
+        t.add_seq(shared + [1000 * (s + 1) + i for i in range(2 * 140 + 1)])   # 141 private chunks each
+    rows = rows_np(t)
+    out = capi.build_tables(rows, t.n_seqs, c, 1, partition, seg, strm, n_heads=4, n_cus=8)
+    plan = out["plan"]
+    check_plan(rows, t.n_seqs, c, plan, 1, partition)
+    for items in (plan["shared_items"], plan["stream_items"]):
+        if len(items):
+            assert items[:, 3].min() >= 1 and items[:, 3].max() <= 64
