@@ -105,9 +105,11 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     }
     // Segment length.  A shared workgroup is a dependent chain of about 2 us per 64 tokens
     // (4 us in the wide form), overlapped with the streaming workgroups of the same launch, so
-    // a segment may take a good part of the step's expected duration (bytes at ~6.4 TB/s) but
-    // not more; longer segments mean fewer partial rows to write and merge, which matters
-    // most when a chunk covers many sequences.
+    // A shared workgroup may run for a good part of the step's expected duration (bytes at
+    // ~6.4 TB/s) but must not outlast it.  Long segments mean fewer workgroups (each pays its
+    // start-up and final merge once), fewer partial rows to write and merge, and fewer slots
+    // taken from the streaming workgroups; measured per 64-token tile, unloaded: ~1.4 us for a
+    // 32-row item, ~2 us for a wide one, and up to twice that next to streaming workgroups.
     int64_t all_tokens = 0;
     for (int i = 0; i < n_rows; i++) {
         all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
@@ -116,9 +118,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     auto seg_chunks_for = [&](int n_covered) {
         if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
         const bool wide = n_covered >= kWideMin;
-        const double tiles = wide ? 0.5 * step_us / 4.0 : 0.4 * step_us / 2.0;
-        const int n_tiles = std::clamp(static_cast<int>(tiles), 4, 32);  // 64-token tiles
-        return std::max(1, n_tiles * 64 / chunk_size);
+        const int n_tiles = std::clamp(static_cast<int>(0.3 * step_us), 4, wide ? 64 : 32);  // 64-token tiles
+        return std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
     };
 
     std::vector<int32_t> n_parts(n_seqs, 0);  // partial rows handed out per sequence so far
