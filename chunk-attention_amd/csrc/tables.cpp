@@ -103,22 +103,35 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         runs.push_back({ i, j - i });
         i = j;
     }
-    // Segment length.  A shared workgroup is a dependent chain of about 2 us per 64 tokens
-    // (4 us in the wide form), overlapped with the streaming workgroups of the same launch, so
-    // A shared workgroup may run for a good part of the step's expected duration (bytes at
-    // ~6.4 TB/s) but must not outlast it.  Long segments mean fewer workgroups (each pays its
-    // start-up and final merge once), fewer partial rows to write and merge, and fewer slots
-    // taken from the streaming workgroups; measured per 64-token tile, unloaded: ~1.4 us for a
-    // 32-row item, ~2 us for a wide one, and up to twice that next to streaming workgroups.
+    // Segment length.  A shared workgroup may run for a good part of the step's expected
+    // duration (bytes at ~6.4 TB/s) but must not outlast it.  Long segments mean fewer
+    // workgroups (each pays its start-up and final merge once), fewer partial rows to write and
+    // merge, and fewer slots taken from the streaming workgroups; measured per 64-token tile,
+    // unloaded: ~1.4 us for a 32-row item, ~2 us for a wide one, and up to twice that next to
+    // streaming workgroups.  When the step is short but the shared work is not (everything
+    // shared, little to stream), the tile count grows until the shared workgroups fit the
+    // device's slots (two per compute unit) in one go.
     int64_t all_tokens = 0;
     for (int i = 0; i < n_rows; i++) {
         all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
     }
     const double step_us = double(all_tokens) * 4.0 * std::max(params.n_heads, 1) * 128.0 / 6.4e6;
+    auto shared_wgs_with = [&](int n_tiles) {   // shared workgroups if every run used n_tiles per segment
+        int64_t wgs = 0;
+        for (const Run& run : runs) {
+            const int n = rows[run.first_row].seq_end - rows[run.first_row].seq_begin;
+            const int seg = std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
+            const int n_segs = std::max({ 1, (run.count + seg / 2) / seg, ceil_div(run.count, kMaxItemChunks) });
+            wgs += int64_t(n_segs) * ceil_div(n, n >= kWideMin ? kWideRows : kMaxRows) * std::max(params.n_heads, 1);
+        }
+        return wgs;
+    };
+    int base_tiles = std::max(static_cast<int>(0.3 * step_us), 4);
+    while (base_tiles < 32 && shared_wgs_with(base_tiles) > int64_t(2) * params.n_cus) base_tiles++;
     auto seg_chunks_for = [&](int n_covered) {
         if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
         const bool wide = n_covered >= kWideMin;
-        const int n_tiles = std::clamp(static_cast<int>(0.3 * step_us), 4, wide ? 64 : 32);  // 64-token tiles
+        const int n_tiles = std::min(base_tiles, wide ? 64 : 32);  // 64-token tiles
         return std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
     };
 
