@@ -129,9 +129,10 @@ int ca_scatter_kv(ca_ctx* ctx, const void* k, const void* v, int n_tokens, int t
 /* Device copy of one chunk's K and V (reference Chunk::deep_copy, chunk.cpp:93-107). */
 int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
 
-/* Work-list shaping.  0 = choose from the device's compute-unit count.
+/* Work-list shaping.  0 = choose from the device's compute-unit count and the step's size.
  * shared_seg_chunks = 1 gives one partial row set per shared chunk, the granularity of the
- * reference's partial buffers. */
+ * reference's partial buffers.  A work item never holds more than 64 chunks: larger values are
+ * cut down to that (63 for stream_chunks, whose last item may take one chunk more). */
 int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
 
 /* How ca_attention is launched.  0 (default): one launch in which chunk-first and sequence-
