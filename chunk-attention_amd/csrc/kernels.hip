@@ -7,10 +7,11 @@
 //                   first phase (stream_path): a run of one sequence's own chunks is streamed
 //                   at HBM speed (16-byte coalesced loads, fp32 online softmax) into one
 //                   partial row, or straight into the output when nothing else is merged.
-//                   The workgroup that completes the last partial of a (sequence, head)
-//                   merges them and writes the normalised output.
-//   merge_kernel    the same merge as a launch of its own, for the two-call
-//                   chunks-first / sequences-first interface.
+//                   Chunks covering ~100 sequences or more take the row-split wide_path.
+//   merge_kernel    merges the partial rows of every (sequence, head) and writes the normalised
+//                   output: the second launch of a forward.  (In the single-launch schedule the
+//                   decode workgroup that completes the last partial of a (sequence, head) does
+//                   this merge itself.)
 //   append_kernel / scatter_kernel   K/V row writes into the chunk pool.
 //
 // Partial rows live in base-2 units: max holds score*log2(e)/sqrt(d), sums and acc are
@@ -511,7 +512,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 //   of column i.  S^T block = K_blk(16 tokens x 128) . Q^T  -> lane owns scores of tokens
 //   4g..4g+3 for sequence i, which is exactly the B operand of O^T = V^T . P^T (k = 16
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
-//   of the 16 x 128 V block read column-wise.
+//   of the 16 x 128 V block through the LDS transpose read (lds_read_tr).
 // ---------------------------------------------------------------------------------------
 template <int C>
 __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
