@@ -33,7 +33,7 @@ def _run(cmd):
 def build_hip_lib() -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, f) for f in ("kernels.hip", "rotary.hip", "c_api.cpp", "tables.cpp", "prefix_tree.cpp")]
+    srcs = [os.path.join(CSRC, f) for f in ("kernels.hip", "rotary.hip", "norm.hip", "c_api.cpp", "tables.cpp", "prefix_tree.cpp")]
     cmd = [hipcc] + HIP_FLAGS + ["-shared", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
                                   "-o", HIP_LIB] + srcs
     _run(cmd)

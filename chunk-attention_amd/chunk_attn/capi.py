@@ -63,6 +63,10 @@ SIGNATURES = {
                                            ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                            ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                            ctypes.c_void_p]),
+    "ca_rms_norm": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float,
+                                   ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
+    "ca_fused_add_rms_norm": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float,
+                                             ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "ca_rope_append_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                          ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
@@ -270,6 +274,38 @@ def rotary_embedding(positions, query, key, head_size: int, cos_sin_cache, is_ne
                                           cos_sin_cache.data_ptr(), n_tokens, query.shape[-1] // head_size,
                                           key.shape[-1] // head_size, head_size, cos_sin_cache.shape[1],
                                           cos_sin_cache.shape[0], q_stride, k_stride, int(is_neox), stream))
+
+
+def _norm_args(name, tensors, weight):
+    import torch
+    hidden = weight.numel()
+    for t in tensors + [weight]:
+        if t.dtype != torch.float16 or t.device.type != "cuda" or not t.is_contiguous():
+            raise RuntimeError(f"{name}: contiguous fp16 tensors on the GPU only")
+    for t in tensors:
+        if t.shape[-1] != hidden or t.shape != tensors[0].shape:
+            raise RuntimeError(f"{name}: rows must be {hidden} wide and of one shape")
+    return tensors[0].numel() // hidden, hidden
+
+
+def rms_norm(out, input, weight, epsilon: float) -> None:
+    """out = rms_norm(input) * weight on torch fp16 tensors, the reference's
+    `chunk_attn.ops.rms_norm` (python_exports_ops.cpp:16)."""
+    import torch
+    n, hidden = _norm_args("rms_norm", [input, out], weight)
+    with torch.cuda.device(input.device):
+        _check(load().ca_rms_norm(out.data_ptr(), input.data_ptr(), weight.data_ptr(), float(epsilon), n, hidden,
+                                  torch.cuda.current_stream(input.device).cuda_stream))
+
+
+def fused_add_rms_norm(input, residual, weight, epsilon: float) -> None:
+    """In place: residual += input; input = rms_norm(residual) * weight, the reference's
+    `chunk_attn.ops.fused_add_rms_norm` (python_exports_ops.cpp:17)."""
+    import torch
+    n, hidden = _norm_args("fused_add_rms_norm", [input, residual], weight)
+    with torch.cuda.device(input.device):
+        _check(load().ca_fused_add_rms_norm(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), float(epsilon),
+                                            n, hidden, torch.cuda.current_stream(input.device).cuda_stream))
 
 
 def max_chunks_for(memory_mb: int, chunk_size: int, n_heads: int, d_head: int, elem_bytes: int = 2) -> int:

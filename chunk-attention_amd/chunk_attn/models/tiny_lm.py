@@ -24,9 +24,10 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
-        return (xf * self.weight.float()).to(x.dtype)
+        x = x.contiguous()
+        out = torch.empty_like(x)
+        capi.rms_norm(out, x, self.weight.detach(), self.eps)
+        return out
 
 
 class AttentionOnlyLM(nn.Module):

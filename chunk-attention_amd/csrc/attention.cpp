@@ -261,4 +261,40 @@ void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Ten
     if (rc != 0) throw std::runtime_error(ca_last_error());
 }
 
+namespace {
+void check_norm_tensor(const torch::Tensor& t, int64_t hidden, const char* what) {
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat16 && t.is_contiguous(), what,
+                ": contiguous float16 tensors on the GPU only");
+    TORCH_CHECK(t.dim() >= 1 && t.size(-1) == hidden, what, ": rows must be as wide as the weight");
+}
+}  // namespace
+
+void rms_norm(torch::Tensor& out, torch::Tensor& input, torch::Tensor& weight, float epsilon) {
+    const int64_t hidden = weight.numel();
+    check_norm_tensor(weight, hidden, "rms_norm");
+    check_norm_tensor(input, hidden, "rms_norm");
+    check_norm_tensor(out, hidden, "rms_norm");
+    TORCH_CHECK(out.sizes() == input.sizes(), "rms_norm: out and input differ in shape");
+    c10::DeviceGuard guard(input.device());
+    void* st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(input.device().index()).stream();
+    if (ca_rms_norm(out.data_ptr(), input.data_ptr(), weight.data_ptr(), epsilon, input.numel() / hidden,
+                    static_cast<int>(hidden), st) != 0) {
+        throw std::runtime_error(ca_last_error());
+    }
+}
+
+void fused_add_rms_norm(torch::Tensor& input, torch::Tensor& residual, torch::Tensor& weight, float epsilon) {
+    const int64_t hidden = weight.numel();
+    check_norm_tensor(weight, hidden, "fused_add_rms_norm");
+    check_norm_tensor(input, hidden, "fused_add_rms_norm");
+    check_norm_tensor(residual, hidden, "fused_add_rms_norm");
+    TORCH_CHECK(residual.sizes() == input.sizes(), "fused_add_rms_norm: input and residual differ in shape");
+    c10::DeviceGuard guard(input.device());
+    void* st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(input.device().index()).stream();
+    if (ca_fused_add_rms_norm(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), epsilon,
+                              input.numel() / hidden, static_cast<int>(hidden), st) != 0) {
+        throw std::runtime_error(ca_last_error());
+    }
+}
+
 }  // namespace GPT

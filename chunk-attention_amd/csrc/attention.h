@@ -86,4 +86,8 @@ class Attention {
 void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Tensor& key, int head_size,
                       torch::Tensor& cos_sin_cache, bool is_neox);
 
+// The reference's rms_norm / fused_add_rms_norm (cpp/chunk_attn/layernorm_kernels.cu:66-117), fp16.
+void rms_norm(torch::Tensor& out, torch::Tensor& input, torch::Tensor& weight, float epsilon);
+void fused_add_rms_norm(torch::Tensor& input, torch::Tensor& residual, torch::Tensor& weight, float epsilon);
+
 }  // namespace GPT

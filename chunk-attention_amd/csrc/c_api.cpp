@@ -510,6 +510,31 @@ int ca_rotary_embedding(const int64_t* positions, void* query, void* key, const 
     return launch_rc(ca::launch_rotary(r, static_cast<hipStream_t>(stream)), "rotary launch");
 }
 
+namespace {
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+}  // namespace
+
+int ca_rms_norm(void* out, const void* input, const void* weight, float epsilon, int64_t n_tokens,
+                int hidden_size, void* stream) {
+    if (n_tokens < 0 || hidden_size <= 0 || !(epsilon >= 0.f)) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_tokens == 0) return CA_OK;
+    if (!out || !input || !weight) return fail(CA_ERR_INVALID, "null device pointer");
+    const bool vec8 = hidden_size % 8 == 0 && aligned16(out) && aligned16(input) && aligned16(weight);
+    return launch_rc(ca::launch_rms_norm(out, const_cast<void*>(input), nullptr, weight, epsilon, n_tokens,
+                                         hidden_size, vec8, static_cast<hipStream_t>(stream)), "rms_norm launch");
+}
+
+int ca_fused_add_rms_norm(void* input, void* residual, const void* weight, float epsilon, int64_t n_tokens,
+                          int hidden_size, void* stream) {
+    if (n_tokens < 0 || hidden_size <= 0 || !(epsilon >= 0.f)) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_tokens == 0) return CA_OK;
+    if (!input || !residual || !weight) return fail(CA_ERR_INVALID, "null device pointer");
+    if (input == residual) return fail(CA_ERR_INVALID, "input and residual must be different buffers");
+    const bool vec8 = hidden_size % 8 == 0 && aligned16(input) && aligned16(residual) && aligned16(weight);
+    return launch_rc(ca::launch_rms_norm(nullptr, input, residual, weight, epsilon, n_tokens, hidden_size, vec8,
+                                         static_cast<hipStream_t>(stream)), "fused_add_rms_norm launch");
+}
+
 int ca_rope_append_kv(ca_ctx* c, const int64_t* positions, void* q, const void* k, const void* v,
                       const void* cos_sin_cache, int max_position, int rot_dim, int is_neox,
                       int n_seqs, void* stream) {

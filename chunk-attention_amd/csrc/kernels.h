@@ -66,4 +66,11 @@ int launch_rope_append(const LaunchArgs& a, const RotaryArgs& r, const void* k, 
                        const int32_t* seq_len, const int32_t* tail_slot, const int32_t* tail_fill,
                        int n_seqs, hipStream_t st);
 
+// RMS normalisation of fp16 rows ([n_tokens, hidden], contiguous).  residual == nullptr:
+// out = norm(input) * weight.  Otherwise the fused form: residual += input (rounded to fp16),
+// input = norm(residual) * weight, `out` unused.  vec8: hidden % 8 == 0 and all pointers 16-byte
+// aligned.
+int launch_rms_norm(void* out, void* input, void* residual, const void* weight, float epsilon,
+                    int64_t n_tokens, int hidden, bool vec8, hipStream_t st);
+
 }  // namespace ca

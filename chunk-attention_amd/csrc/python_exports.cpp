@@ -70,9 +70,13 @@ PYBIND11_MODULE(chunk_attn_c, m) {
       .def("value", &Attention::value, py::arg("chunk"));
 
     // the reference's chunk_attn.ops module (cpp/chunk_attn/python_exports_ops.cpp:11-19), the part the
-    // decode path's caller uses
+    // decode path's callers use (all three of its operators)
     py::module ops = m.def_submodule("ops", "operators used around the attention call");
     ops.def("rotary_embedding", &GPT::rotary_embedding, py::arg("positions"), py::arg("query"), py::arg("key"),
             py::arg("head_size"), py::arg("cos_sin_cache"), py::arg("is_neox"),
             "Apply GPT-NeoX or GPT-J style rotary embedding to query and key");
+    ops.def("rms_norm", &GPT::rms_norm, py::arg("out"), py::arg("input"), py::arg("weight"), py::arg("epsilon"),
+            "Apply Root Mean Square (RMS) Normalization to the input tensor.");
+    ops.def("fused_add_rms_norm", &GPT::fused_add_rms_norm, py::arg("input"), py::arg("residual"),
+            py::arg("weight"), py::arg("epsilon"), "In-place fused Add and RMS Normalization");
 }

@@ -107,6 +107,17 @@ int ca_rotary_embedding(const int64_t* positions_dev, void* query, void* key,
                         int n_kv_heads, int head_size, int rot_dim, int max_position,
                         int64_t query_stride, int64_t key_stride, int is_neox, void* stream);
 
+/* Replace rms_norm(out, input, weight, epsilon) and fused_add_rms_norm(input, residual, weight,
+ * epsilon) (cpp/chunk_attn/layernorm_kernels.cu:66-117, bound in python_exports_ops.cpp:16-18):
+ * fp16 rows [n_tokens, hidden_size], contiguous, fp32 statistics.
+ *   ca_rms_norm:            out = fp16(x * rsqrt(mean(x^2) + epsilon)) * weight   (out may equal input)
+ *   ca_fused_add_rms_norm:  residual = fp16(input + residual);
+ *                           input = fp16(residual * rsqrt(mean((input + residual)^2) + epsilon)) * weight */
+int ca_rms_norm(void* out, const void* input, const void* weight, float epsilon, int64_t n_tokens,
+                int hidden_size, void* stream);
+int ca_fused_add_rms_norm(void* input, void* residual, const void* weight, float epsilon,
+                          int64_t n_tokens, int hidden_size, void* stream);
+
 /* The decode step of the reference's attention layer
  * (src/chunk_attn/models/llama_hf/modeling_llama.py:62,91-95: rotary_embedding on the new
  * query/key rows, then append_token -> append_kv) as one launch: q [n_seqs, n_heads, d_head]
