@@ -78,7 +78,8 @@ struct ca_ctx {
 
     std::vector<ca::ChunkRow> rows;  // rows of the last refresh (to rebuild for another partition)
     int n_seqs = 0;
-    ca::RefTables ref;
+    mutable ca::RefTables ref;  // reference-form tables of `rows`: use ref_tables(), never directly
+    mutable bool ref_valid = false;
     ca::Plan plan;
 
     // device tables: one blob, uploaded from one of two pinned staging buffers
@@ -213,6 +214,15 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
     c->partition = partition;
     return CA_OK;
+}
+
+// Reference-form tables of the rows the context holds, built on first use after a refresh.
+const ca::RefTables& ref_tables(const ca_ctx* c) {
+    if (!c->ref_valid) {
+        ca::build_ref_tables(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, c->tpp_threshold, &c->ref);
+        c->ref_valid = true;
+    }
+    return c->ref;
 }
 
 int check_ready(ca_ctx* c, const void* q, int n_seqs) {
@@ -358,7 +368,7 @@ int ca_refresh_kernel_context(ca_ctx* c, const ca_chunk_row* rows, int n_rows, i
         c->rows.resize(n_rows);
         if (n_rows) std::memcpy(c->rows.data(), rows, sizeof(ca_chunk_row) * n_rows);
         c->n_seqs = n_seqs;
-        ca::build_ref_tables(c->rows.data(), n_rows, n_seqs, c->C, c->tpp_threshold, &c->ref);
+        c->ref_valid = false;  // reference-form tables are for inspection: built when asked for
         if (int rc = build_and_upload(c, 0, static_cast<hipStream_t>(stream))) return rc;
         c->delta_tokens = 0;
         c->valid = true;
@@ -612,17 +622,20 @@ int ca_ctx_set_schedule(ca_ctx* c, int mode) {
 
 int ca_ctx_plan_info(const ca_ctx* c, ca_plan_info* info) {
     if (!c || !info) return fail(CA_ERR_INVALID, "bad argument");
-    info->n_seqs = c->n_seqs;
-    info->n_chunks = c->ref.n_chunks;
-    info->n_shared_chunks = c->ref.n_shared;
-    info->ref_partial_rows = c->ref.partial_rows;
-    info->max_seq_n_chunks = c->ref.max_seq_n_chunks;
-    info->n_shared_items = static_cast<int>(c->plan.shared_items.size());
-    info->n_stream_items = static_cast<int>(c->plan.stream_items.size());
-    info->n_part_rows = c->plan.n_part_rows;
-    info->shared_tokens = c->plan.shared_tokens;
-    info->stream_tokens = c->plan.stream_tokens;
-    return CA_OK;
+    return guarded([&]() -> int {
+        const ca::RefTables& ref = ref_tables(c);
+        info->n_seqs = c->n_seqs;
+        info->n_chunks = ref.n_chunks;
+        info->n_shared_chunks = ref.n_shared;
+        info->ref_partial_rows = ref.partial_rows;
+        info->max_seq_n_chunks = ref.max_seq_n_chunks;
+        info->n_shared_items = static_cast<int>(c->plan.shared_items.size());
+        info->n_stream_items = static_cast<int>(c->plan.stream_items.size());
+        info->n_part_rows = c->plan.n_part_rows;
+        info->shared_tokens = c->plan.shared_tokens;
+        info->stream_tokens = c->plan.stream_tokens;
+        return CA_OK;
+    });
 }
 
 int ca_ctx_ref_tables(const ca_ctx* c, int32_t* final_idx, int32_t* slots, int32_t* begins,
@@ -632,14 +645,17 @@ int ca_ctx_ref_tables(const ca_ctx* c, int32_t* final_idx, int32_t* slots, int32
     auto copy = [](int32_t* dst, const std::vector<int32_t>& src) {
         if (dst && !src.empty()) std::memcpy(dst, src.data(), src.size() * 4);
     };
-    copy(final_idx, c->ref.final_idx);
-    copy(slots, c->ref.slots);
-    copy(begins, c->ref.begins);
-    copy(ends, c->ref.ends);
-    copy(offsets, c->ref.offsets);
-    copy(seq_n_tokens, c->ref.seq_n_tokens);
-    copy(seq_chunk_map, c->ref.seq_chunk_map);
-    return CA_OK;
+    return guarded([&]() -> int {
+        const ca::RefTables& ref = ref_tables(c);
+        copy(final_idx, ref.final_idx);
+        copy(slots, ref.slots);
+        copy(begins, ref.begins);
+        copy(ends, ref.ends);
+        copy(offsets, ref.offsets);
+        copy(seq_n_tokens, ref.seq_n_tokens);
+        copy(seq_chunk_map, ref.seq_chunk_map);
+        return CA_OK;
+    });
 }
 
 int ca_ctx_export_partials(ca_ctx* c, float* maxs, float* sums, float* attns, void* stream) {
@@ -669,10 +685,11 @@ int ca_ctx_export_partials(ca_ctx* c, float* maxs, float* sums, float* attns, vo
                 chunk++;
                 prev_slot_first = it.slot_first;
             }
-            if (chunk >= c->ref.n_shared) return fail(CA_ERR_STATE, "shared items do not match the shared chunks");
-            const int off = c->ref.offsets[chunk];
-            const int b = c->ref.begins[chunk];
-            const int n = c->ref.ends[chunk] - b;
+            const ca::RefTables& ref = ref_tables(c);
+            if (chunk >= ref.n_shared) return fail(CA_ERR_STATE, "shared items do not match the shared chunks");
+            const int off = ref.offsets[chunk];
+            const int b = ref.begins[chunk];
+            const int n = ref.ends[chunk] - b;
             for (int h = 0; h < c->H; h++) {
                 for (int r = 0; r < it.n_rows; r++) {
                     const int s = it.seq_begin + r;
