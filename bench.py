@@ -145,6 +145,29 @@ def side_costs(attn, w, torch, capi):
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
 
 
+def decode_loop(w, torch, capi, synth, seed, unique_tokens):
+    """The configuration's decode loop on a fresh cache: per step one append_token (K/V rows of
+    every sequence into the tails, chunk fill -> reserve -> table rebuild when a tail is full)
+    and one forward, through the torch-tensor interface; wall-clock per step."""
+    lw = synth.two_level_workload(w.name + "-loop", 8, 8, w.chunk_size, 1024, 512, unique_tokens,
+                                  n_heads=w.n_heads, append_steps=w.append_steps)
+    attn = build_cache(lw, torch, capi, seed)
+    q = torch.from_numpy(lw.q(seed)).to("cuda:0")
+    kv = [tuple(torch.from_numpy(a).to("cuda:0") for a in lw.append_kv(t, seed)) for t in range(lw.append_steps)]
+    toks = [lw.append_tokens(t) for t in range(lw.append_steps)]
+    attn.forward(q)
+    torch.cuda.synchronize()
+    new_chunks, t0 = 0, time.perf_counter()
+    for t in range(lw.append_steps):
+        new_chunks += attn.append_token(toks[t], kv[t][0], kv[t][1])
+        attn.forward(q)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / lw.append_steps
+    return {"steps": lw.append_steps, "unique_tokens_at_start": unique_tokens, "us_per_step": round(us, 1),
+            "chunks_added": int(new_chunks),
+            "note": "append_token + forward per step through the ctypes/torch interface, host work included"}
+
+
 def cpu_baseline(attn, q_np, budget_s, torch):
     """The CPU restatement of the reference's MKL path on the same cache contents (fp16 values
     widened to fp32), timed on this machine's host cores."""
@@ -268,6 +291,10 @@ def main() -> int:
     }
 
     result["per_step_side_costs"] = side_costs(attn, w, torch, capi)
+    if args.config == 3:
+        # the two-level configuration's 32 decode steps: as given (tails never fill) and with
+        # 100 private tokens, where every tail fills at step 28 (reserve + table rebuild)
+        result["decode_loop"] = [decode_loop(w, torch, capi, synth, args.seed, u) for u in (128, 100)]
 
     if not args.no_paged:
         pw = synth.paged_variant(w)
