@@ -154,11 +154,6 @@ __device__ __forceinline__ float reduce_rows16(float (&v)[NV], int j) {
 }
 
 // ---------------------------------------------------------------------------------------
-// stream_kernel: grid = n_items * H workgroups.  Wave w of a workgroup takes chunks
-// w, w+4, ... of the item; a chunk is read as 64-token sub-tiles (32 for chunk_size 32).
-// Lane l = 16*g + j reads, for load i, the 16 bytes at offset 1024*i + 16*l of a sub-tile:
-// row 4*i + g, dims 8*j..8*j+7, so every load instruction covers 1 KiB of contiguous memory.
-// ---------------------------------------------------------------------------------------
 // Every wave fetches the slot ids of its item's chunks (at most 64: kMaxItemChunks) with one
 // load, chunk k into lane k, when it starts.  Looking a slot up in memory right before the
 // chunk's K/V loads would put a dependent round trip in front of every tile, and waiting for
@@ -279,6 +274,13 @@ union __attribute__((aligned(16))) DecodeLds {
     WidePathLds wd;
 };
 
+// ---------------------------------------------------------------------------------------
+// stream_path: an item = a run of one sequence's own chunks.  Wave w of the workgroup takes
+// tiles w, w+4, ... of the item (a tile = one chunk, or two chunks at chunk size 32) and reads
+// them as 64-token sub-tiles.  Lane l = 16*g + j reads, for load i, the 16 bytes at offset
+// 1024*i + 16*l of a sub-tile: row 4*i + g, dims 8*j..8*j+7, so every load instruction covers
+// 1 KiB of contiguous memory and 32 of them (K, then V) are in flight per wave.
+// ---------------------------------------------------------------------------------------
 template <int C>
 __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, StreamPathLds& sm) {
@@ -292,9 +294,15 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     const int32_t* __restrict__ slots = A.slots;
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
-    constexpr int SUB = (C < 64) ? C : 64;  // tokens per sub-tile
-    constexpr int NL = SUB / 4;             // 16-byte loads per lane per sub-tile
-    constexpr int NSUB = C / SUB;
+    // A wave works on 64-token sub-tiles: one chunk at chunk size 64, half a chunk at 128, two
+    // consecutive chunks of the item at 32 (their loads go out together, so a wave has the same
+    // 32 KiB in flight at every chunk size).
+    constexpr int SUB = 64;                        // tokens per sub-tile
+    constexpr int NL = SUB / 4;                    // 16-byte loads per lane per sub-tile
+    constexpr int CPT = (C < SUB) ? SUB / C : 1;   // chunks per tile
+    constexpr int NSUB = (C > SUB) ? C / SUB : 1;  // sub-tiles per tile
+    constexpr int LPC = NL / CPT;                  // loads per lane that one chunk supplies
+    static_assert(C == 32 || C == 64 || C == 128, "chunk sizes of the decode kernels");
 
     const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
@@ -363,32 +371,51 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     };
     bool tried = !can_fold;
 
-    for (int t = w; t < it.n_chunks; t += NW) {
+    for (int t = w * CPT; t < it.n_chunks; t += NW * CPT) {
         int valid = len - (it.pos0 + t) * C;
         if (valid <= 0) break;  // chunks are in path order: everything after is empty too
-        valid = valid < C ? valid : C;
-        const int slot = chunk_slot(slotv, t);
-        const size_t base = (size_t(slot) * H + h) * size_t(C) * D;
+        // tokens of this tile: bounded by the sequence's end and by the item's last chunk (the
+        // sequence may go on in another item)
+        const int n_here = (it.n_chunks - t < CPT) ? it.n_chunks - t : CPT;
+        valid = valid < n_here * C ? valid : n_here * C;
+        size_t base[CPT];
+#pragma unroll
+        for (int cc = 0; cc < CPT; cc++) {
+            const int tc = (cc < n_here) ? t + cc : t;  // a missing second chunk is never loaded
+            base[cc] = (size_t(chunk_slot(slotv, tc)) * H + h) * size_t(C) * D;
+        }
 #pragma unroll
         for (int sub = 0; sub < NSUB; sub++) {
             const int vsub = valid - sub * SUB;  // valid rows in this sub-tile
             if (vsub <= 0) break;
             const bool masked = vsub < SUB;
-            const uint4* kp = reinterpret_cast<const uint4*>(kpool + base + size_t(sub) * SUB * D) + l;
-            const uint4* vp = reinterpret_cast<const uint4*>(vpool + base + size_t(sub) * SUB * D) + l;
+            // load i of the sub-tile: 1 KiB at offset (i % LPC) KiB of chunk i / LPC
+            const uint4* kp[CPT];
+            const uint4* vp[CPT];
+#pragma unroll
+            for (int cc = 0; cc < CPT; cc++) {
+                kp[cc] = reinterpret_cast<const uint4*>(kpool + base[cc] + size_t(sub) * SUB * D) + l;
+                vp[cc] = reinterpret_cast<const uint4*>(vpool + base[cc] + size_t(sub) * SUB * D) + l;
+            }
             uint4 kr[NL], vr[NL];
             if (!masked) {
 #pragma unroll
-                for (int i = 0; i < NL; i++) kr[i] = A.stream_nt ? nt_load16(kp + 64 * i) : kp[64 * i];
+                for (int i = 0; i < NL; i++) {
+                    const uint4* p = kp[i / LPC] + 64 * (i % LPC);
+                    kr[i] = A.stream_nt ? nt_load16(p) : *p;
+                }
 #pragma unroll
-                for (int i = 0; i < NL; i++) vr[i] = A.stream_nt ? nt_load16(vp + 64 * i) : vp[64 * i];
+                for (int i = 0; i < NL; i++) {
+                    const uint4* p = vp[i / LPC] + 64 * (i % LPC);
+                    vr[i] = A.stream_nt ? nt_load16(p) : *p;
+                }
             } else {
                 // rows past the end of the sequence hold stale data: never read into the math
 #pragma unroll
                 for (int i = 0; i < NL; i++) {
                     const bool ok = 4 * i + g < vsub;
-                    kr[i] = ok ? kp[64 * i] : make_uint4(0, 0, 0, 0);
-                    vr[i] = ok ? vp[64 * i] : make_uint4(0, 0, 0, 0);
+                    kr[i] = ok ? kp[i / LPC][64 * (i % LPC)] : make_uint4(0, 0, 0, 0);
+                    vr[i] = ok ? vp[i / LPC][64 * (i % LPC)] : make_uint4(0, 0, 0, 0);
                 }
             }
             float sc[NL];

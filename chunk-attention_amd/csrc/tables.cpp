@@ -192,10 +192,12 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     if (stream_chunks <= 0) {
         // four waves per workgroup each take whole chunks, so prefer multiples of four;
         // shrink towards four when there would be too few workgroups to fill the device
+        // (never below one 64-token tile per wave: 256 tokens, and four chunks)
         const int per_wg_tokens = 512;
-        stream_chunks = std::max(4, per_wg_tokens / chunk_size);
+        const int min_chunks = std::max(4, 256 / chunk_size);
+        stream_chunks = std::max(min_chunks, per_wg_tokens / chunk_size);
         const int64_t target = int64_t(2) * params.n_cus;
-        while (stream_chunks > 4 &&
+        while (stream_chunks > min_chunks &&
                (stream_chunk_total / stream_chunks) * std::max(params.n_heads, 1) < target) {
             stream_chunks /= 2;
         }
