@@ -93,6 +93,7 @@ struct ca_ctx {
     size_t off_shared = 0, off_stream = 0, off_slots = 0, off_seq_len = 0, off_part_ptr = 0,
            off_tail_slot = 0, off_tail_fill = 0;
     int schedule = 0;  // 0: partial-producing launch + merge launch; 1: one launch, last finisher merges
+    int plan_schedule = 0;  // schedule the current plan was built for
 
     float* part = nullptr;
     size_t part_cap = 0;  // bytes
@@ -142,6 +143,7 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     // its K/V there again on the next step, and plain loads top out near 6.3 TB/s against
     // 7.2 TB/s for loads with the non-temporal hint (measured with a bare read kernel): stream
     // the private chunks around the cache then.  Smaller working sets keep plain loads.
+    a.stream_per_wave = c->plan.stream_per_wave;
     a.stream_nt = (int64_t(c->plan.stream_tokens) + c->plan.shared_tokens) * 4 * c->H * c->d > (int64_t(256) << 20);
     return a;
 }
@@ -161,6 +163,7 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     pp.stream_chunks = c->stream_chunks;
     pp.n_heads = c->H;
     pp.n_cus = c->n_cus;
+    pp.allow_per_wave = c->schedule == 0;  // the single-launch schedule synchronises workgroups
     ca::build_plan(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, pp, &c->plan);
     ca::Plan& p = c->plan;
 
@@ -213,6 +216,7 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     if (int rc = ensure_dev(reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
     if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
     c->partition = partition;
+    c->plan_schedule = c->schedule;
     return CA_OK;
 }
 
@@ -393,7 +397,7 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
     if (n_seqs == 0) return CA_OK;
     return guarded([&]() -> int {
         hipStream_t st = static_cast<hipStream_t>(stream);
-        if (partition != c->partition) {
+        if (partition != c->partition || c->schedule != c->plan_schedule) {
             if (int rc = build_and_upload(c, partition, st)) return rc;
         }
         if (!c->timing) return run_fused(c, q, out, st);

@@ -31,6 +31,9 @@ struct LaunchArgs {
     // forward streams more than the last-level cache holds: the data cannot be found there
     // again, and without the hint it only displaces what could be.
     bool stream_nt = false;
+    // Every wave of a stream workgroup takes a stream item of its own (four consecutive items per
+    // workgroup): set by the plan when there are many short runs.  Not with fuse_merge.
+    bool stream_per_wave = false;
 };
 
 // All return 0, -1 for an unsupported shape, or a positive hipError_t.

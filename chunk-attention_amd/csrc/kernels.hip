@@ -190,6 +190,8 @@ struct DecodeArgs {
     int H;
     float scale_log2;
     int fuse_merge;  // 1: the last workgroup to finish a (sequence, head) merges its partials
+    int n_stream_items;   // stream items in the list
+    int stream_per_wave;  // 1: every wave of a stream workgroup takes an item of its own (needs fuse_merge 0)
     int stream_nt;   // 1: private chunks are read with the non-temporal hint (see LaunchArgs)
 };
 
@@ -281,7 +283,9 @@ union __attribute__((aligned(16))) DecodeLds {
 // 1024*i + 16*l of a sub-tile: row 4*i + g, dims 8*j..8*j+7, so every load instruction covers
 // 1 KiB of contiguous memory and 32 of them (K, then V) are in flight per wave.
 // ---------------------------------------------------------------------------------------
-template <int C>
+// PER_WAVE: the wave works alone on its own item (all tiles, no cross-wave combine, no barrier):
+// the form for many short runs, where a workgroup per run would spend its life starting up.
+template <int C, bool PER_WAVE>
 __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, StreamPathLds& sm) {
     WorkItem it;  // header only: the inline slots are read from global memory where needed
@@ -323,7 +327,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     // folds rows w, w+4, ... of the list straight into its running softmax state, so nothing
     // is published and nothing remains to merge.  Each wave tries once after its first tile,
     // when the row loads hide behind the streaming; the rest happens at the end.
-    const bool can_fold = A.fuse_merge && it.part_row >= 0;
+    const bool can_fold = !PER_WAVE && A.fuse_merge && it.part_row >= 0;
     const int p0 = (it.part_row >= 0) ? A.part_ptr[seq] : 0;
     const int p1 = (it.part_row >= 0) ? A.part_ptr[seq + 1] : 0;
     const int own = p0 + it.part_row;  // this workgroup's partial row
@@ -371,7 +375,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     };
     bool tried = !can_fold;
 
-    for (int t = w * CPT; t < it.n_chunks; t += NW * CPT) {
+    for (int t = (PER_WAVE ? 0 : w) * CPT; t < it.n_chunks; t += (PER_WAVE ? 1 : NW) * CPT) {
         int valid = len - (it.pos0 + t) * C;
         if (valid <= 0) break;  // chunks are in path order: everything after is empty too
         // tokens of this tile: bounded by the sequence's end and by the item's last chunk (the
@@ -477,6 +481,24 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     for (int e = 0; e < 8; e++) {
         acc[e] += shfl_xor(acc[e], 16);
         acc[e] += shfl_xor(acc[e], 32);
+    }
+    if constexpr (PER_WAVE) {
+        // lanes of group 0 hold dims 8j..8j+7 of the wave's (= the item's) result
+        if (g == 0) {
+            if (it.part_row < 0) {
+                const float r = l_wave > 0.f ? 1.f / l_wave : 0.f;
+                h8 o8;
+#pragma unroll
+                for (int e = 0; e < 8; e++) o8[e] = half_t(acc[e] * r);
+                *reinterpret_cast<h8*>(A.out + (size_t(seq) * H + h) * D + 8 * j) = o8;
+            } else {
+                float* own_row = A.part + (size_t(own) * H + h) * PART_STRIDE;
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) part_store2(own_row + 4 + 8 * j + e, acc[e], acc[e + 1]);
+                if (j == 0) part_store2(own_row, m_run, l_wave);
+            }
+        }
+        return;
     }
     if (g == 0) {
 #pragma unroll
@@ -994,7 +1016,13 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
         }
     } else {
         const int sid = bid - A.n_shared_wgs;
-        stream_path<C>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
+        if (A.stream_per_wave) {
+            // four consecutive items per workgroup, one per wave, same head
+            const int item = 4 * (sid / A.H) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            if (item < A.n_stream_items) stream_path<C, true>(A, A.stream_items + item, sid % A.H, lds.st);
+        } else {
+            stream_path<C, false>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
+        }
     }
 }
 
@@ -1086,17 +1114,23 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.H = a.H;
     d.scale_log2 = a.scale_log2;
     d.fuse_merge = 0;
+    d.n_stream_items = 0;
+    d.stream_per_wave = 0;
     d.stream_nt = a.stream_nt ? 1 : 0;
     return d;
 }
 
 int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, bool fuse_merge,
                   hipStream_t st) {
-    const int64_t wgs = int64_t(n_shared_items + n_stream_items) * a.H;
+    if (a.stream_per_wave && fuse_merge) return -1;  // waves on their own never meet at a barrier
+    const int stream_groups = a.stream_per_wave ? (n_stream_items + NW - 1) / NW : n_stream_items;
+    const int64_t wgs = int64_t(n_shared_items + stream_groups) * a.H;
     if (wgs <= 0) return 0;
     DecodeArgs d = decode_args(a);
     d.n_shared_wgs = n_shared_items * a.H;
     d.fuse_merge = fuse_merge ? 1 : 0;
+    d.n_stream_items = n_stream_items;
+    d.stream_per_wave = a.stream_per_wave ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
     switch (a.C) {
         case 32: hipLaunchKernelGGL(decode_kernel<32>, grid, block, 0, st, d); break;

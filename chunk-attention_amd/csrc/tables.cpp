@@ -236,6 +236,18 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         }
     }
 
+    // Many short runs (a long shared prompt, a few private tokens each): a workgroup per run
+    // would spend most of its life starting up, and only some of its waves would have a tile.
+    // When every item is at most three 64-token tiles and there are enough of them to fill the
+    // device at one item per wave, each wave takes an item of its own.
+    {
+        int max_tiles = 0;
+        for (const WorkItem& it : p.stream_items) max_tiles = std::max(max_tiles, ceil_div(it.n_chunks * chunk_size, 64));
+        const int64_t tasks = int64_t(p.stream_items.size()) * std::max(params.n_heads, 1);
+        p.stream_per_wave = params.allow_per_wave && !p.stream_items.empty() && max_tiles <= 3 &&
+                            tasks >= int64_t(3) * 2 * params.n_cus;
+    }
+
     // a sequence whose only partial comes from a stream item needs no merge: that item
     // writes the final output itself and its partial row is dropped from the merge list
     for (auto& it : p.stream_items) {

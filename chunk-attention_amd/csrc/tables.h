@@ -68,6 +68,7 @@ struct PlanParams {
     int stream_chunks = 0;      // max chunks per stream item, 0 = choose from n_cus
     int n_heads = 32;
     int n_cus = 256;
+    bool allow_per_wave = true;  // the launch schedule can run stream items one per wave
 };
 
 constexpr int kMaxRows = 32;    // sequences per shared work item (M tile)
@@ -79,6 +80,7 @@ struct Plan {
     int n_seqs = 0;
     int n_part_rows = 0;
     int max_parts_per_seq = 0;
+    bool stream_per_wave = false;  // stream items are short and many: one per wave, four per workgroup
     int64_t shared_tokens = 0;   // physical tokens attended chunk-first (per head)
     int64_t stream_tokens = 0;   // tokens attended by stream items (per head, at build time)
     std::vector<WorkItem> shared_items;
