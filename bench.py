@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0
 def build_cache(w, torch, capi, seed=0, tpp_threshold=1):
     import numpy as np
     dev = torch.device("cuda:0")
-    need = sum(w.seq_len(s) // w.chunk_size + 2 for s in range(w.n_seqs)) + 8
+    need = sum(w.seq_len(s) // w.chunk_size + 2 for s in range(w.n_seqs)) + 2048 // w.chunk_size + 10   # + room for side_costs
     per_chunk = w.chunk_size * w.n_heads * w.d_head * 2 * 2
     memory_mb = -(-need * per_chunk // (1 << 20))
     attn = capi.Attention(n_heads=w.n_heads, d_head=w.d_head, chunk_size=w.chunk_size, memory_mb=memory_mb,
@@ -140,7 +140,25 @@ def side_costs(attn, w, torch, capi):
                                 True, w.n_seqs, stream)
     torch.cuda.synchronize()
     fused_us = (time.perf_counter() - t0) * 1e6 / reps
+    # prefill copy-in: a 2048-token sequence that shares nothing (every K/V row is scattered into
+    # fresh chunks), inserted and removed again; wall clock with a device sync per insertion
+    T = 2048
+    pk = torch.zeros((T, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    toks = [-(10 ** 9) - i for i in range(T)]
+    idx = attn.add_seq(toks, pk, pk)
+    attn.remove_seq(idx)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        idx = attn.add_seq(toks, pk, pk)
+        torch.cuda.synchronize()
+        attn.remove_seq(idx)
+    add_us = (time.perf_counter() - t0) * 1e6 / 5
+    attn.refresh_kernel_context()
+    torch.cuda.synchronize()
+    copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
     return {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
+            "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
 
