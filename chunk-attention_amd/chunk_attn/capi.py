@@ -35,7 +35,8 @@ class PlanInfo(ctypes.Structure):
                 ("n_shared_chunks", ctypes.c_int32), ("ref_partial_rows", ctypes.c_int32),
                 ("max_seq_n_chunks", ctypes.c_int32), ("n_shared_items", ctypes.c_int32),
                 ("n_stream_items", ctypes.c_int32), ("n_part_rows", ctypes.c_int32),
-                ("shared_tokens", ctypes.c_int64), ("stream_tokens", ctypes.c_int64)]
+                ("shared_tokens", ctypes.c_int64), ("stream_tokens", ctypes.c_int64),
+                ("stream_per_wave", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 # name -> (restype, argtypes); every symbol include/chunk_attn_hip.h declares

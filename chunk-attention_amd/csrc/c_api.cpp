@@ -638,6 +638,8 @@ int ca_ctx_plan_info(const ca_ctx* c, ca_plan_info* info) {
         info->n_part_rows = c->plan.n_part_rows;
         info->shared_tokens = c->plan.shared_tokens;
         info->stream_tokens = c->plan.stream_tokens;
+        info->stream_per_wave = c->plan.stream_per_wave ? 1 : 0;
+        info->reserved = 0;
         return CA_OK;
     });
 }
@@ -771,6 +773,8 @@ int ca_tables_info(const ca_tables* t, ca_plan_info* info) {
     info->n_part_rows = t->plan.n_part_rows;
     info->shared_tokens = t->plan.shared_tokens;
     info->stream_tokens = t->plan.stream_tokens;
+    info->stream_per_wave = t->plan.stream_per_wave ? 1 : 0;
+    info->reserved = 0;
     return CA_OK;
 }
 

@@ -178,6 +178,8 @@ typedef struct ca_plan_info {
     int32_t n_part_rows;
     int64_t shared_tokens;      /* physical tokens attended chunk-first */
     int64_t stream_tokens;      /* tokens streamed per sequence (when the tables were built) */
+    int32_t stream_per_wave;    /* 1: stream items run one per wave, four per workgroup (many short runs) */
+    int32_t reserved;
 } ca_plan_info;
 int ca_ctx_plan_info(const ca_ctx* ctx, ca_plan_info* info);
 

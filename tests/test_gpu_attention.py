@@ -295,3 +295,38 @@ def test_long_paths_split_into_items_of_at_most_64_chunks(c):
             tables = capi.build_tables(attn.get_chunks(), B, c, 1, partition, seg, strm, n_heads=H)
             for items in (tables["plan"]["shared_items"], tables["plan"]["stream_items"]):
                 assert len(items) == 0 or items[:, 3].max() <= 64
+
+
+def test_many_short_private_runs_one_item_per_wave():
+    """Enough short private runs (sequences x heads) make the plan run stream items one per
+    wave.  Ragged runs of one to three chunks, sequences that end exactly on a chunk boundary,
+    appends that fill tails and open new chunks: every step must match the oracle, in the
+    default schedule (per wave) and in the single-launch schedule (which must not use it)."""
+    rng = np.random.default_rng(60)
+    H, c, B = 32, 32, 56
+    P = 2 * c
+    sk, sv = rand16(rng, P, H, 128), rand16(rng, P, H, 128)
+    attn = make_attention(H, c, 2 + B * 6)
+    for s in range(B):
+        U = [5, c, c + 7, 2 * c, 2 * c + 9, 1][s % 6]
+        k, v = rand16(rng, P + U, H, 128), rand16(rng, P + U, H, 128)
+        k[:P], v[:P] = sk, sv
+        assert attn.add_seq(list(range(P)) + [1_000_000 * (s + 1) + i for i in range(U)], to_dev(k), to_dev(v)) == s
+    q = rand16(rng, B, H, 128)
+    attn.refresh_kernel_context()
+    assert attn.ctx.plan_info().stream_per_wave == 1
+    for step in range(c + 3):
+        if step % 8 == 0 or step > c - 2:
+            want = oracle_output(attn, q, exact=True)
+            assert_close(attn.forward(to_dev(q)), want)
+            assert_close(attn.forward(to_dev(q), 2), want)      # everything streamed
+        k1, v1 = rand16(rng, B, H, 128), rand16(rng, B, H, 128)
+        attn.append_token([7_000_000 + 64 * step + s for s in range(B)], to_dev(k1), to_dev(v1))
+    want = oracle_output(attn, q, exact=True)
+    assert_close(attn.forward(to_dev(q)), want)
+    attn.ctx.set_schedule(1)
+    assert_close(attn.forward(to_dev(q)), want)
+    assert attn.ctx.plan_info().stream_per_wave == 0
+    attn.ctx.set_schedule(0)
+    assert_close(attn.forward(to_dev(q)), want)
+    assert attn.ctx.plan_info().stream_per_wave == 1
