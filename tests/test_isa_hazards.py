@@ -85,10 +85,13 @@ def readers(insts, start, count, dst):
 @pytest.mark.skipif(not shutil.which(HIPCC) and not os.path.exists(HIPCC), reason="hipcc not available")
 def test_no_branch_between_matrix_op_and_first_reader(tmp_path):
     asm = tmp_path / "kernels.s"
-    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
-                           "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
-                           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.dirname(SRC), "-S",
-                           "--cuda-device-only", "-o", str(asm), SRC], stderr=subprocess.DEVNULL)
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("ca_build", os.path.join(ROOT, "chunk-attention_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)           # the library's own compiler flags
+    flags = [f for f in build.HIP_FLAGS if f != "-fPIC"]
+    subprocess.check_call([HIPCC] + flags + ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.dirname(SRC), "-S",
+                                             "--cuda-device-only", "-o", str(asm), SRC], stderr=subprocess.DEVNULL)
     insts = parse(asm)
     labels = {lab: i for i, (lab, mn, _) in enumerate(insts) if lab}
     n_mfma, problems = 0, []
