@@ -139,11 +139,11 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.C = c->C;
     a.d = c->d;
     a.scale_log2 = 1.4426950408889634f / std::sqrt(static_cast<float>(c->d));
+    a.stream_per_wave = c->plan.stream_per_wave;
     // 256 MiB of Infinity Cache on this part.  A forward that attends more than that cannot find
     // its K/V there again on the next step, and plain loads top out near 6.3 TB/s against
     // 7.2 TB/s for loads with the non-temporal hint (measured with a bare read kernel): stream
     // the private chunks around the cache then.  Smaller working sets keep plain loads.
-    a.stream_per_wave = c->plan.stream_per_wave;
     a.stream_nt = (int64_t(c->plan.stream_tokens) + c->plan.shared_tokens) * 4 * c->H * c->d > (int64_t(256) << 20);
     return a;
 }
