@@ -157,7 +157,27 @@ def side_costs(attn, w, torch, capi):
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
     copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
-    return {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
+    # the layer's norm operators on a prefill-sized activation [2048, H*d] (launches timed with
+    # events on the current stream): rms_norm reads and writes the rows once, the fused form reads
+    # and writes both the activation and the residual
+    hidden = w.n_heads * w.d_head
+    x = torch.randn((T, hidden), device="cuda:0").half()
+    res, y = torch.randn_like(x), torch.empty_like(x)
+    wt = torch.ones(hidden, dtype=torch.float16, device="cuda:0")
+    norm = {}
+    for name, fn, passes in (("rms_norm", lambda: capi.rms_norm(y, x, wt, 1e-6), 2),
+                             ("fused_add_rms_norm", lambda: capi.fused_add_rms_norm(x, res, wt, 1e-6), 4)):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        norm[name + "_2048x%d_us" % hidden] = round(us, 1)
+        norm[name + "_GBps"] = round(passes * T * hidden * 2 / us / 1e3, 1)
+    return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
