@@ -157,11 +157,13 @@ def side_costs(attn, w, torch, capi):
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
     copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
-    # the layer's norm operators on a prefill-sized activation [2048, H*d] (launches timed with
-    # events on the current stream): rms_norm reads and writes the rows once, the fused form reads
-    # and writes both the activation and the residual
+    # the layer's norm operators on a prefill batch of 16384 rows of H*d (128 MiB per tensor, so
+    # that a launch outlasts the host's ~10 us per call; launch trains timed with events on the
+    # current stream): rms_norm reads and writes the rows once, the fused form reads and writes
+    # both the activation and the residual
     hidden = w.n_heads * w.d_head
-    x = torch.randn((T, hidden), device="cuda:0").half()
+    TN = 16384
+    x = torch.randn((TN, hidden), device="cuda:0").half()
     res, y = torch.randn_like(x), torch.empty_like(x)
     wt = torch.ones(hidden, dtype=torch.float16, device="cuda:0")
     norm = {}
@@ -175,8 +177,8 @@ def side_costs(attn, w, torch, capi):
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / reps
-        norm[name + "_2048x%d_us" % hidden] = round(us, 1)
-        norm[name + "_GBps"] = round(passes * T * hidden * 2 / us / 1e3, 1)
+        norm[name + "_%dx%d_us" % (TN, hidden)] = round(us, 1)
+        norm[name + "_GBps"] = round(passes * TN * hidden * 2 / us / 1e3, 1)
     return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),

@@ -32,6 +32,39 @@ __device__ __forceinline__ float block_sum(float v, float* sm) {
 }
 
 // VEC = 8: rows are multiples of 8 elements and 16-byte aligned; VEC = 1: any row length.
+// With VEC = 8 a thread keeps the first KEEP pieces it reads (rows of up to KEEP * 2048 elements
+// entirely) in registers between the two passes, so the row is read from memory once; longer rows
+// re-read the rest.
+constexpr int KEEP = 4;
+
+// One 8-element piece of the first pass: returns its contribution to the sum of squares and
+// leaves in x what the second pass normalises (with ADD: the rounded sum, also written to residual).
+template <bool ADD>
+__device__ __forceinline__ float first_pass8(h8& x, half_t* __restrict__ residual_piece) {
+    float ss = 0.f;
+    if constexpr (ADD) {
+        const h8 r = *reinterpret_cast<const h8*>(residual_piece);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float s = float(x[e]) + float(r[e]);
+            ss += s * s;
+            x[e] = half_t(s);
+        }
+        *reinterpret_cast<h8*>(residual_piece) = x;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) ss += float(x[e]) * float(x[e]);
+    }
+    return ss;
+}
+
+__device__ __forceinline__ h8 second_pass8(const h8 x, const h8 w, float inv) {
+    h8 y;
+#pragma unroll
+    for (int e = 0; e < 8; e++) y[e] = half_t(float(x[e]) * inv) * w[e];
+    return y;
+}
+
 template <int VEC, bool ADD>
 __global__ __launch_bounds__(WG) void rms_norm_kernel(half_t* __restrict__ out, half_t* __restrict__ input,
                                                       half_t* __restrict__ residual,
@@ -39,24 +72,41 @@ __global__ __launch_bounds__(WG) void rms_norm_kernel(half_t* __restrict__ out, 
                                                       int hidden) {
     __shared__ float sm[4];
     const size_t row = size_t(blockIdx.x) * hidden;
+    const half_t* src = ADD ? residual : input;
+    half_t* dst = ADD ? input : out;
     float ss = 0.f;
-    for (int idx = threadIdx.x * VEC; idx < hidden; idx += WG * VEC) {
-        if constexpr (VEC == 8) {
+    if constexpr (VEC == 8) {
+        h8 kept[KEEP];
+#pragma unroll
+        for (int it = 0; it < KEEP; it++) {  // the loads of all kept pieces go out together
+            const int idx = (threadIdx.x + it * WG) * 8;
+            if (idx < hidden) kept[it] = *reinterpret_cast<const h8*>(input + row + idx);
+        }
+#pragma unroll
+        for (int it = 0; it < KEEP; it++) {
+            const int idx = (threadIdx.x + it * WG) * 8;
+            if (idx < hidden) ss += first_pass8<ADD>(kept[it], ADD ? residual + row + idx : nullptr);
+        }
+        for (int idx = (threadIdx.x + KEEP * WG) * 8; idx < hidden; idx += WG * 8) {
             h8 x = *reinterpret_cast<const h8*>(input + row + idx);
-            if constexpr (ADD) {
-                const h8 r = *reinterpret_cast<const h8*>(residual + row + idx);
+            ss += first_pass8<ADD>(x, ADD ? residual + row + idx : nullptr);
+        }
+        const float inv = __builtin_amdgcn_rsqf(block_sum(ss, sm) / float(hidden) + epsilon);
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float s = float(x[e]) + float(r[e]);
-                    ss += s * s;
-                    x[e] = half_t(s);
-                }
-                *reinterpret_cast<h8*>(residual + row + idx) = x;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) ss += float(x[e]) * float(x[e]);
+        for (int it = 0; it < KEEP; it++) {
+            const int idx = (threadIdx.x + it * WG) * 8;
+            if (idx < hidden) {
+                *reinterpret_cast<h8*>(dst + row + idx) =
+                  second_pass8(kept[it], *reinterpret_cast<const h8*>(weight + idx), inv);
             }
-        } else {
+        }
+        // (with ADD, a thread re-reads here only what it wrote above itself)
+        for (int idx = (threadIdx.x + KEEP * WG) * 8; idx < hidden; idx += WG * 8) {
+            *reinterpret_cast<h8*>(dst + row + idx) =
+              second_pass8(*reinterpret_cast<const h8*>(src + row + idx), *reinterpret_cast<const h8*>(weight + idx), inv);
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < hidden; idx += WG) {
             float s = float(input[row + idx]);
             if constexpr (ADD) {
                 s += float(residual[row + idx]);
@@ -64,20 +114,8 @@ __global__ __launch_bounds__(WG) void rms_norm_kernel(half_t* __restrict__ out, 
             }
             ss += s * s;
         }
-    }
-    // (with ADD, a thread re-reads below only what it wrote above itself)
-    const float inv = __builtin_amdgcn_rsqf(block_sum(ss, sm) / float(hidden) + epsilon);
-    const half_t* src = ADD ? residual : input;
-    half_t* dst = ADD ? input : out;
-    for (int idx = threadIdx.x * VEC; idx < hidden; idx += WG * VEC) {
-        if constexpr (VEC == 8) {
-            const h8 x = *reinterpret_cast<const h8*>(src + row + idx);
-            const h8 w = *reinterpret_cast<const h8*>(weight + idx);
-            h8 y;
-#pragma unroll
-            for (int e = 0; e < 8; e++) y[e] = half_t(float(x[e]) * inv) * w[e];
-            *reinterpret_cast<h8*>(dst + row + idx) = y;
-        } else {
+        const float inv = __builtin_amdgcn_rsqf(block_sum(ss, sm) / float(hidden) + epsilon);
+        for (int idx = threadIdx.x; idx < hidden; idx += WG) {
             dst[row + idx] = half_t(float(src[row + idx]) * inv) * weight[idx];
         }
     }
