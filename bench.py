@@ -179,6 +179,19 @@ def side_costs(attn, w, torch, capi):
         us = e0.elapsed_time(e1) * 1e3 / reps
         norm[name + "_%dx%d_us" % (TN, hidden)] = round(us, 1)
         norm[name + "_GBps"] = round(passes * TN * hidden * 2 / us / 1e3, 1)
+    # the rotary operator on the same batch: q and k rows of H*d, read and written once
+    kq = torch.randn((TN, hidden), device="cuda:0").half()
+    posn = torch.arange(TN, device="cuda:0", dtype=torch.int64) % 8192
+    capi.rotary_embedding(posn, x, kq, w.d_head, cache, True)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        capi.rotary_embedding(posn, x, kq, w.d_head, cache, True)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    norm["rotary_embedding_%dx%d_us" % (TN, hidden)] = round(us, 1)
+    norm["rotary_embedding_GBps"] = round(4 * TN * hidden * 2 / us / 1e3, 1)
     return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),

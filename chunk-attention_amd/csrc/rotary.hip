@@ -69,6 +69,57 @@ __global__ __launch_bounds__(WG) void rotary_kernel(const int64_t* __restrict__ 
     row[yi] = half_t(rot_elem(y, x, c, s, false));
 }
 
+// The same operator for rows made of whole 16-byte pieces (head_size, strides and, NeoX style,
+// rot_dim / 2 multiples of 8; GPT-J style rot_dim a multiple of 8; 16-byte aligned pointers): one
+// thread rotates 8 pairs (NeoX: the pieces at r0 and r0 + rot_dim/2) or 4 pairs (GPT-J: one
+// piece), so every load and store moves 16 bytes per lane.  Same arithmetic as rotary_kernel.
+template <bool IS_NEOX>
+__global__ __launch_bounds__(WG) void rotary_vec_kernel(const int64_t* __restrict__ positions,
+                                                        half_t* __restrict__ query,
+                                                        half_t* __restrict__ key,
+                                                        const half_t* __restrict__ cache,
+                                                        int64_t n_tokens, int n_heads, int n_kv_heads,
+                                                        int head_size, int rot_dim, int max_position,
+                                                        int64_t query_stride, int64_t key_stride) {
+    const int embed = rot_dim / 2;
+    const int units = IS_NEOX ? embed / 8 : rot_dim / 8;  // work units per head
+    const int64_t per_token = int64_t(n_heads + n_kv_heads) * units;
+    const int64_t idx = int64_t(blockIdx.x) * WG + threadIdx.x;
+    if (idx >= n_tokens * per_token) return;
+    const int64_t token = idx / per_token;
+    const int rem = static_cast<int>(idx % per_token);
+    const int head = rem / units, u = rem % units;
+    half_t* row = (head < n_heads) ? query + token * query_stride + int64_t(head) * head_size
+                                   : key + token * key_stride + int64_t(head - n_heads) * head_size;
+    const half_t* cs = cache + clamp_pos(positions[token], max_position) * rot_dim;
+    if constexpr (IS_NEOX) {
+        const int r0 = 8 * u;
+        h8 x = *reinterpret_cast<const h8*>(row + r0);
+        h8 y = *reinterpret_cast<const h8*>(row + embed + r0);
+        const h8 c8 = *reinterpret_cast<const h8*>(cs + r0);
+        const h8 s8 = *reinterpret_cast<const h8*>(cs + embed + r0);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float xf = float(x[e]), yf = float(y[e]), c = float(c8[e]), sn = float(s8[e]);
+            x[e] = half_t(rot_elem(xf, yf, c, sn, true));
+            y[e] = half_t(rot_elem(yf, xf, c, sn, false));
+        }
+        *reinterpret_cast<h8*>(row + r0) = x;
+        *reinterpret_cast<h8*>(row + embed + r0) = y;
+    } else {
+        h8 v = *reinterpret_cast<const h8*>(row + 8 * u);
+        const h4 c4 = *reinterpret_cast<const h4*>(cs + 4 * u);
+        const h4 s4 = *reinterpret_cast<const h4*>(cs + embed + 4 * u);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float xf = float(v[2 * e]), yf = float(v[2 * e + 1]), c = float(c4[e]), sn = float(s4[e]);
+            v[2 * e] = half_t(rot_elem(xf, yf, c, sn, true));
+            v[2 * e + 1] = half_t(rot_elem(yf, xf, c, sn, false));
+        }
+        *reinterpret_cast<h8*>(row + 8 * u) = v;
+    }
+}
+
 // One thread owns 8 consecutive elements of one (sequence, head) row of q, k or v:
 // units [0, n) are query rows, [n, 2n) key rows, [2n, 3n) value rows, n = n_seqs * H * d/8.
 // Requires d % 8 == 0 and, NeoX style, rot_dim % 16 == 0 (the pairing partner is then another
@@ -139,13 +190,35 @@ __global__ __launch_bounds__(WG) void rope_append_kernel(
     } while (0)
 
 int launch_rotary(const RotaryArgs& r, hipStream_t st) {
+    half_t* q = static_cast<half_t*>(r.query);
+    half_t* k = static_cast<half_t*>(r.key);
+    const half_t* cache = static_cast<const half_t*>(r.cos_sin_cache);
+    auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool pieces = r.head_size % 8 == 0 && r.rot_dim % (r.is_neox ? 16 : 8) == 0 &&
+                        r.query_stride % 8 == 0 && r.key_stride % 8 == 0 && aligned16(q) && aligned16(k) &&
+                        aligned16(cache);
+    if (pieces) {
+        const int units = r.is_neox ? r.rot_dim / 16 : r.rot_dim / 8;
+        const int64_t total = r.n_tokens * int64_t(r.n_heads + r.n_kv_heads) * units;
+        if (total <= 0) return 0;
+        if (total > int64_t(0x7fffffff) * WG) return -1;
+        const dim3 grid(static_cast<unsigned>((total + WG - 1) / WG)), block(WG);
+        if (r.is_neox) {
+            hipLaunchKernelGGL(rotary_vec_kernel<true>, grid, block, 0, st, r.positions, q, k, cache, r.n_tokens,
+                               r.n_heads, r.n_kv_heads, r.head_size, r.rot_dim, r.max_position,
+                               r.query_stride, r.key_stride);
+        } else {
+            hipLaunchKernelGGL(rotary_vec_kernel<false>, grid, block, 0, st, r.positions, q, k, cache, r.n_tokens,
+                               r.n_heads, r.n_kv_heads, r.head_size, r.rot_dim, r.max_position,
+                               r.query_stride, r.key_stride);
+        }
+        CA_LAUNCH_CHECK();
+        return 0;
+    }
     const int64_t total = r.n_tokens * int64_t(r.n_heads + r.n_kv_heads) * (r.rot_dim / 2);
     if (total <= 0) return 0;
     if (total > int64_t(0x7fffffff) * WG) return -1;
     const dim3 grid(static_cast<unsigned>((total + WG - 1) / WG)), block(WG);
-    half_t* q = static_cast<half_t*>(r.query);
-    half_t* k = static_cast<half_t*>(r.key);
-    const half_t* cache = static_cast<const half_t*>(r.cos_sin_cache);
     if (r.is_neox) {
         hipLaunchKernelGGL(rotary_kernel<true>, grid, block, 0, st, r.positions, q, k, cache, r.n_tokens,
                            r.n_heads, r.n_kv_heads, r.head_size, r.rot_dim, r.max_position,

@@ -26,7 +26,7 @@ def exact_rotation(pos, rows, head_size, cache, is_neox):
 
 
 @pytest.mark.parametrize("is_neox", [True, False])
-@pytest.mark.parametrize("head_size,rot_dim,n_heads,n_kv", [(128, 128, 32, 32), (64, 32, 5, 1), (16, 16, 2, 2), (6, 2, 3, 2)])
+@pytest.mark.parametrize("head_size,rot_dim,n_heads,n_kv", [(128, 128, 32, 32), (64, 32, 5, 1), (16, 16, 2, 2), (6, 2, 3, 2), (64, 24, 3, 3), (20, 12, 2, 1)])
 def test_rotary_embedding(is_neox, head_size, rot_dim, n_heads, n_kv):
     rng = np.random.default_rng(11)
     n, max_pos = 37, 500
