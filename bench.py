@@ -154,6 +154,19 @@ def side_costs(attn, w, torch, capi):
         torch.cuda.synchronize()
         attn.remove_seq(idx)
     add_us = (time.perf_counter() - t0) * 1e6 / 5
+    # the copy-in launch by itself: the same rows scattered again into the chunks of one such
+    # sequence (a launch train between events; nothing else owns those chunks)
+    idx = attn.add_seq(toks, pk, pk)
+    own = [int(r[0]) for r in attn.get_chunks() if r[2] == idx and r[3] == idx + 1 and r[1] > 0]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    attn.ctx.scatter_kv(pk.data_ptr(), pk.data_ptr(), T, 0, own, stream)
+    e0.record()
+    for _ in range(reps):
+        attn.ctx.scatter_kv(pk.data_ptr(), pk.data_ptr(), T, 0, own, stream)
+    e1.record()
+    torch.cuda.synchronize()
+    scatter_us = e0.elapsed_time(e1) * 1e3 / reps
+    attn.remove_seq(idx)
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
     copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
@@ -194,6 +207,7 @@ def side_costs(attn, w, torch, capi):
     norm["rotary_embedding_GBps"] = round(4 * TN * hidden * 2 / us / 1e3, 1)
     return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
+            "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
 
