@@ -211,10 +211,13 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
 
     const size_t part_bytes = std::max<size_t>(size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4, 256);
     if (int rc = ensure_dev(reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
-    // completion counters start at zero; each forward leaves them at zero again
-    const int n_counters = std::max(c->n_seqs * c->H, 1);
-    if (int rc = ensure_dev(reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
-    if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
+    // completion counters (single-launch schedule only; a change of schedule rebuilds the plan and
+    // comes through here): they start at zero, and each forward leaves them at zero again
+    if (c->schedule != 0) {
+        const int n_counters = std::max(c->n_seqs * c->H, 1);
+        if (int rc = ensure_dev(reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
+        if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
+    }
     c->partition = partition;
     c->plan_schedule = c->schedule;
     return CA_OK;
