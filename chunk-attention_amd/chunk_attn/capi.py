@@ -108,6 +108,10 @@ SIGNATURES = {
     "ca_tree_used_chunks": (ctypes.c_int, [ctypes.c_void_p]),
     "ca_tree_version": (ctypes.c_uint64, [ctypes.c_void_p]),
     "ca_tree_tails": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p]),
+    "ca_tree_duplicate": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, c_i32_p, ctypes.c_int,
+                                         c_int_p]),
+    "ca_tree_append_completion": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, c_i32_p, ctypes.c_int, c_i32_p,
+                                                 ctypes.c_int, c_int_p, c_i32_p]),
     "ca_tree_dump": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p, c_i32_p,
                                     ctypes.c_int, c_int_p]),
 }
@@ -188,6 +192,31 @@ class Tree:
         n = ctypes.c_int()
         _check(self._lib.ca_tree_append_token(self._h, ptr, len(tokens), ctypes.byref(n)))
         return n.value
+
+    def duplicate(self, seq_idx: int, copies: int) -> List[Tuple[int, int]]:
+        """`copies` more sequences identical to seq_idx right after it; returns the (source slot,
+        destination slot) pairs whose K/V chunks the caller copies."""
+        if copies < 1:
+            return []
+        pairs = (ctypes.c_int32 * (2 * copies))()
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_duplicate(self._h, seq_idx, copies, pairs, copies, ctypes.byref(n)))
+        return [(pairs[2 * i], pairs[2 * i + 1]) for i in range(n.value)]
+
+    def append_completion(self, seq_idx: int, tokens: Sequence[int]):
+        """One beam-search step on seq_idx.  Returns (copy pairs, targets): chunk copies to make
+        first, then targets[i] = (slot, row) of the K/V row of candidate i (sequence seq_idx + i)."""
+        n_tok = len(tokens)
+        if n_tok < 1:
+            return [], []
+        arr, ptr = _i32(tokens)
+        pairs = (ctypes.c_int32 * (2 * max(n_tok - 1, 1)))()
+        targets = (ctypes.c_int32 * (2 * n_tok))()
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_append_completion(self._h, seq_idx, ptr, n_tok, pairs, n_tok - 1, ctypes.byref(n),
+                                                   targets))
+        return ([(pairs[2 * i], pairs[2 * i + 1]) for i in range(n.value)],
+                [(targets[2 * i], targets[2 * i + 1]) for i in range(n_tok)])
 
     def get_chunks(self) -> np.ndarray:
         """[n_rows, 4] int32: slot, n_tokens, seq_begin, seq_end in get_chunks order."""
@@ -591,6 +620,31 @@ class Attention:
         self.tree.append_token(tokens)
         self.ctx.delta_tokens = self.ctx.delta_tokens + 1
         return n_new
+
+    def duplicate(self, seq_idx: int, copies: int) -> None:
+        """Beam search: `copies` more sequences identical to seq_idx, right after it (reference
+        attention.cpp:287-313); each owns a device copy of the tail chunk."""
+        for src, dst in self.tree.duplicate(seq_idx, copies):
+            self.ctx.copy_chunk(src, dst, self._stream())
+        self.ctx.invalidate()
+
+    def append_completion(self, seq_idx: int, tokens: Sequence[int], k, v) -> int:
+        """One beam-search step (reference attention.cpp:227-261): candidate 0 continues seq_idx
+        with tokens[0] and row 0 of k/v, candidates 1.. become sequences seq_idx+1.. ."""
+        n = len(tokens)
+        if n < 1:
+            return seq_idx
+        k = self._check_kv(k, n, "k")
+        v = self._check_kv(v, n, "v")
+        pairs, targets = self.tree.append_completion(seq_idx, tokens)
+        for src, dst in pairs:
+            self.ctx.copy_chunk(src, dst, self._stream())
+        kp, vp = self.pool_views()
+        for i, (slot, row) in enumerate(targets):       # same stream: after the copies
+            kp[slot, :, row].copy_(k[i])
+            vp[slot, :, row].copy_(v[i])
+        self.ctx.invalidate()
+        return seq_idx
 
     def forward(self, q, partition: int = 0):
         import torch

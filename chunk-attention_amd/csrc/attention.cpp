@@ -193,23 +193,26 @@ void Attention::duplicate(int seq_idx, int copies) {
 }
 
 int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::Tensor k, torch::Tensor v) {
-    // beam search step (reference attention.cpp:216-261): candidate 0 continues the sequence,
+    // beam search step (reference attention.cpp:227-261): candidate 0 continues the sequence,
     // candidates 1.. become copies of its tail inserted right after it, each with its own token
     const int n = static_cast<int>(tokens.size());
     if (n < 1) return seq_idx;
     if (seq_idx < 0 || seq_idx >= tree_->n_seqs()) throw std::out_of_range("no such sequence");
     k = checked_kv(k, n, "k");
     v = checked_kv(v, n, "v");
-    tree_->reserve();
-    if (n > 1) duplicate(seq_idx, n - 1);
-    // row i of k/v becomes the next token of sequence seq_idx + i
+    std::vector<std::pair<int, int>> pairs;
+    std::vector<PrefixTree::RowTarget> rows;
+    tree_->append_completion(seq_idx, tokens, &pairs, &rows);
     c10::DeviceGuard guard(t_options_.device());
-    const auto& tails = tree_->tails();
+    for (const auto& [src, dst] : pairs) check(ca_copy_chunk(ctx_, src, dst, stream()));
+    // row i of k/v is the new token of sequence seq_idx + i (same stream: after the copies)
+    const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
+    auto chunk_view = [&](torch::Tensor& storage, int slot) {
+        return storage.narrow(0, chunk_elems * slot, chunk_elems).view({ n_heads_, chunk_size_, d_head_ });
+    };
     for (int i = 0; i < n; i++) {
-        Chunk* tail = tails[seq_idx + i];
-        key(tail).select(1, tail->n_tokens()).copy_(k[i]);
-        value(tail).select(1, tail->n_tokens()).copy_(v[i]);
-        tail->append_tokens(tokens, i, i + 1);
+        chunk_view(key_storage_, rows[i].slot).select(1, rows[i].row).copy_(k[i]);
+        chunk_view(value_storage_, rows[i].slot).select(1, rows[i].row).copy_(v[i]);
     }
     ca_ctx_invalidate(ctx_);  // sequence lengths changed under the device tables
     return seq_idx;

@@ -913,6 +913,48 @@ int ca_tree_n_seqs(const ca_tree* t) { return t ? t->tree.n_seqs() : 0; }
 int ca_tree_used_chunks(const ca_tree* t) { return t ? t->tree.allocator().used_chunks() : 0; }
 uint64_t ca_tree_version(const ca_tree* t) { return t ? t->tree.version() : 0; }
 
+int ca_tree_duplicate(ca_tree* t, int seq_idx, int copies, int32_t* copy_pairs, int cap_pairs, int* n_pairs) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    if (n_pairs) *n_pairs = 0;
+    if (copies < 1) return CA_OK;
+    if (!copy_pairs || cap_pairs < copies) return fail(CA_ERR_INVALID, "copy_pairs holds fewer than `copies` pairs");
+    return guarded([&]() -> int {
+        std::vector<std::pair<int, int>> pairs;
+        t->tree.duplicate(seq_idx, copies, &pairs);
+        for (size_t i = 0; i < pairs.size(); i++) {
+            copy_pairs[2 * i] = pairs[i].first;
+            copy_pairs[2 * i + 1] = pairs[i].second;
+        }
+        if (n_pairs) *n_pairs = static_cast<int>(pairs.size());
+        return CA_OK;
+    });
+}
+
+int ca_tree_append_completion(ca_tree* t, int seq_idx, const int32_t* tokens, int n_tokens,
+                              int32_t* copy_pairs, int cap_pairs, int* n_pairs, int32_t* targets) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    if (n_pairs) *n_pairs = 0;
+    if (n_tokens < 0 || (n_tokens > 0 && (!tokens || !targets))) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_tokens > 1 && (!copy_pairs || cap_pairs < n_tokens - 1)) {
+        return fail(CA_ERR_INVALID, "copy_pairs holds fewer than n_tokens - 1 pairs");
+    }
+    return guarded([&]() -> int {
+        std::vector<std::pair<int, int>> pairs;
+        std::vector<GPT::PrefixTree::RowTarget> rows;
+        t->tree.append_completion(seq_idx, std::vector<int>(tokens, tokens + n_tokens), &pairs, &rows);
+        for (size_t i = 0; i < pairs.size(); i++) {
+            copy_pairs[2 * i] = pairs[i].first;
+            copy_pairs[2 * i + 1] = pairs[i].second;
+        }
+        for (size_t i = 0; i < rows.size(); i++) {
+            targets[2 * i] = rows[i].slot;
+            targets[2 * i + 1] = rows[i].row;
+        }
+        if (n_pairs) *n_pairs = static_cast<int>(pairs.size());
+        return CA_OK;
+    });
+}
+
 int ca_tree_tails(const ca_tree* t, int32_t* slots, int cap, int* n) {
     if (!t) return fail(CA_ERR_INVALID, "null tree");
     const auto& tails = t->tree.tails();

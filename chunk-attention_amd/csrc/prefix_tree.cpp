@@ -241,6 +241,9 @@ void PrefixTree::duplicate(int seq_idx, int copies, std::vector<std::pair<int, i
     if (copies < 1) return;
     Chunk* tail = at(seq_idx);
     if (tail->parent == nullptr) throw std::runtime_error("duplicate: empty tree");
+    if (copies > alloc_.max_chunks() - alloc_.used_chunks()) {
+        throw std::runtime_error("ChunkAllocator: capacity reached");  // before anything changes
+    }
     for (Chunk* node = tail->parent; node != nullptr; node = node->parent) node->n_seqs += copies;
     auto& sib = tail->parent->children;
     int pos = static_cast<int>(std::find(sib.begin(), sib.end(), tail) - sib.begin()) + 1;
@@ -252,6 +255,50 @@ void PrefixTree::duplicate(int seq_idx, int copies, std::vector<std::pair<int, i
         tails_.insert(tails_.begin() + seq_idx + 1 + i, copy);
         if (copy_slots) copy_slots->emplace_back(tail->slot_, copy->slot_);
     }
+    version_++;
+}
+
+void PrefixTree::append_completion(int seq_idx, const std::vector<int>& tokens,
+                                   std::vector<std::pair<int, int>>* copy_slots,
+                                   std::vector<RowTarget>* targets) {
+    const int n = static_cast<int>(tokens.size());
+    if (seq_idx < 0 || seq_idx >= static_cast<int>(tails_.size())) {
+        throw std::out_of_range("append_completion: no such sequence");
+    }
+    if (targets) targets->assign(n, RowTarget{ -1, -1 });
+    if (n < 1) return;
+    Chunk* chunk = tails_[seq_idx];
+    // chunks this step takes, so that running out of them leaves the tree as it was
+    const bool was_full = chunk->full();
+    const bool fills = (was_full ? 0 : chunk->n_tokens()) + 1 == chunk_size_;  // this token fills the tail
+    const int need = (was_full ? 1 : 0) + (n - 1) * (fills ? 2 : 1) + (fills ? 1 : 0);
+    if (need > alloc_.max_chunks() - alloc_.used_chunks()) {
+        throw std::runtime_error("ChunkAllocator: capacity reached");
+    }
+    if (was_full) {
+        chunk = chunk->add_child(alloc_.allocate());
+        tails_[seq_idx] = chunk;
+    }
+    if (n > 1) {
+        for (Chunk* node = chunk->parent; node != nullptr; node = node->parent) node->n_seqs += n - 1;
+        auto& sib = chunk->parent->children;
+        int pos = static_cast<int>(std::find(sib.begin(), sib.end(), chunk) - sib.begin()) + 1;
+        for (int i = 1; i < n; i++) {
+            Chunk* copy = alloc_.allocate();
+            copy->tokens = chunk->tokens;  // reference chunk.cpp:93-107 (deep copy of a tail)
+            copy->n_seqs = 1;
+            if (copy_slots) copy_slots->emplace_back(chunk->slot_, copy->slot_);
+            if (targets) (*targets)[i] = RowTarget{ copy->slot_, copy->n_tokens() };
+            copy->append_tokens(tokens, i, i + 1);
+            chunk->parent->insert_child(pos++, copy);
+            Chunk* tail = copy;
+            if (copy->full()) tail = copy->add_child(alloc_.allocate());  // full chunks are not tails
+            tails_.insert(tails_.begin() + seq_idx + i, tail);
+        }
+    }
+    if (targets) (*targets)[0] = RowTarget{ chunk->slot_, chunk->n_tokens() };
+    chunk->append_tokens(tokens, 0, 1);
+    if (chunk->full()) tails_[seq_idx] = chunk->add_child(alloc_.allocate());
     version_++;
 }
 

@@ -101,12 +101,26 @@ class PrefixTree {
     void append_token_ids(const std::vector<int>& tokens);
     // reference attention.cpp:342-372 (pre-order, children visited last-to-first)
     std::vector<ChunkInfo> get_chunks() const;
-    // reference attention.cpp:200-214
+    // reference attention.cpp:211-226
     Chunk* at(int seq_idx) const;
     // tree half of reference attention.cpp:287-313: `copies` more sequences identical to
     // seq_idx, inserted right after it.  Each new tail's K/V must be copied from the
     // source tail by the caller (src slot -> dst slot pairs are appended to `copy_slots`).
     void duplicate(int seq_idx, int copies, std::vector<std::pair<int, int>>* copy_slots);
+    // tree half of reference attention.cpp:227-261, one beam-search step on sequence seq_idx:
+    // candidate 0 continues the sequence with tokens[0]; candidates 1.. become copies of its tail,
+    // inserted right after it, each continued with its own token; a tail that fills up gets its
+    // empty child at once.  The caller copies K/V chunk src -> dst for every pair appended to
+    // `copy_slots`, then writes candidate i's K/V row at (*targets)[i] (sequence seq_idx + i).
+    // Differences from the reference, which leaves the tree inconsistent: the ancestors'
+    // sequence counts and the tail list are updated, and a full tail (which the reference only
+    // asserts against) first gets its empty child.
+    struct RowTarget {
+        int slot;
+        int row;
+    };
+    void append_completion(int seq_idx, const std::vector<int>& tokens,
+                           std::vector<std::pair<int, int>>* copy_slots, std::vector<RowTarget>* targets);
 
     Chunk* root() { return &root_; }
     const std::vector<Chunk*>& tails() const { return tails_; }

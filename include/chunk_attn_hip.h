@@ -264,6 +264,22 @@ int ca_tree_get_chunks(const ca_tree* tree, ca_chunk_row* rows, int cap, int* n_
 int ca_tree_n_seqs(const ca_tree* tree);
 int ca_tree_used_chunks(const ca_tree* tree);
 uint64_t ca_tree_version(const ca_tree* tree);
+/* Tree half of reference Attention::duplicate (attention.cpp:287-313): `copies` more sequences
+ * identical to seq_idx, inserted right after it (indices seq_idx+1 ..).  Every new sequence
+ * shares the path and owns a copy of the tail chunk: copy_pairs (capacity cap_pairs >= copies
+ * pairs) receives (source slot, destination slot) per copy, for ca_copy_chunk.  Unlike the
+ * reference, the tail list is updated as well. */
+int ca_tree_duplicate(ca_tree* tree, int seq_idx, int copies, int32_t* copy_pairs, int cap_pairs,
+                      int* n_pairs);
+/* Tree half of reference Attention::append_completion (attention.cpp:227-261), one beam-search
+ * step: candidate 0 continues sequence seq_idx with tokens[0]; candidates 1 .. n_tokens-1 become
+ * copies of its tail right after it, each continued with its own token.  copy_pairs (capacity
+ * cap_pairs >= n_tokens - 1) receives the (source, destination) slots to copy first; targets
+ * [n_tokens][2] receives (slot, row) where candidate i's K/V row belongs (sequence seq_idx + i).
+ * Unlike the reference, sequence counts and the tail list stay consistent, and a full tail gets
+ * its empty child first instead of tripping an assertion. */
+int ca_tree_append_completion(ca_tree* tree, int seq_idx, const int32_t* tokens, int n_tokens,
+                              int32_t* copy_pairs, int cap_pairs, int* n_pairs, int32_t* targets);
 /* slot of the tail chunk of every sequence, in sequence order (reference tails()) */
 int ca_tree_tails(const ca_tree* tree, int32_t* slots, int cap, int* n);
 /* Pre-order dump (children first-to-last) of the whole tree for structure checks: per node

@@ -12,7 +12,10 @@ Pinned by (see tests/test_oracle_tree.py):
   * the literal expectations of the reference's own tests
     (tests/test_chunk_attn_cpu.py:24-175 add, :177-215 append, :267-303 remove),
   * the hand-worked table example for the tree after those six inserts,
-  * a brute-force model that recomputes sharing from the raw token lists.
+  * a brute-force model that recomputes sharing from the raw token lists,
+  * for the beam-search operations (duplicate, append_completion), which the reference's own
+    test suite skips: the list-of-token-lists model (every sequence's root-to-tail tokens), the
+    tree invariants, and hand-worked trees.
 """
 from __future__ import annotations
 
@@ -199,6 +202,103 @@ class PrefixTree:
             node = parent
         del self.tails[seq_idx]
         self.valid = False
+
+    # attention.cpp:211-226
+    def at(self, seq_idx: int) -> Chunk:
+        if not 0 <= seq_idx < self.root.n_seqs:
+            raise IndexError("no such sequence")
+        chunk = self.root
+        start = 0
+        while chunk.children:
+            for child in chunk.children:
+                end = start + child.n_seqs
+                if start <= seq_idx < end:
+                    chunk = child
+                    break
+                start = end
+        return chunk
+
+    def _copy_of_tail(self, tail: Chunk) -> Chunk:
+        """chunk_allocator.cpp:87-91 -> Chunk::deep_copy (chunk.cpp:93-107): tokens copied,
+        n_seqs = 1; copying a chunk with children is refused."""
+        if tail.children:
+            raise RuntimeError("Copy a non tailing chunk is forbidden")
+        copy = self.alloc.allocate()
+        copy.tokens = list(tail.tokens)
+        copy.n_seqs = 1
+        return copy
+
+    # attention.cpp:287-313.  Every node above the tail counts `copies` more sequences, and
+    # `copies` deep copies of the tail go in right after it (Chunk::insert_child,
+    # chunk.cpp:115-120).  The reference stops there, leaving tails() and the kernel context
+    # stale; here the tail list gains the copies at seq_idx+1.. and the context is
+    # invalidated.  Returns the (source slot, copy slot) pairs whose K/V must be copied.
+    def duplicate(self, seq_idx: int, copies: int) -> List[Tuple[int, int]]:
+        if copies < 1:
+            return []
+        tail = self.at(seq_idx)
+        node = tail.parent
+        while node is not None:
+            node.n_seqs += copies
+            node = node.parent
+        distance = tail.parent.children.index(tail) + 1
+        pairs = []
+        for i in range(copies):
+            copy = self._copy_of_tail(tail)
+            tail.parent.children.insert(distance, copy)
+            copy.parent = tail.parent
+            distance += 1
+            self.tails.insert(seq_idx + 1 + i, copy)
+            pairs.append((tail.slot, copy.slot))
+        self.valid = False
+        return pairs
+
+    # attention.cpp:227-261, one beam-search step: candidates 1.. are copies of the tail (taken
+    # before candidate 0's token is appended) that continue with their own token and go in right
+    # after it; then the tail takes tokens[0]; a chunk that fills up gets its empty child at once
+    # ("make sure full chunks are not the tails").  The reference leaves the ancestors' n_seqs
+    # and tails() untouched, which makes the tree inconsistent, and asserts that the tail is not
+    # full; here the counts and the tail list follow, and a full tail first gets its empty child
+    # (what reserve() would do for it).  Returns (copy pairs, [(slot, row) of each candidate's
+    # K/V row]); candidate i is sequence seq_idx + i afterwards.
+    def append_completion(self, seq_idx: int, tokens: Sequence[int]):
+        n = len(tokens)
+        if n < 1:
+            return [], []
+        chunk = self.at(seq_idx)
+        need = (1 if chunk.full() else 0)
+        fills = (0 if chunk.full() else chunk.n_tokens) + 1 == self.chunk_size
+        need += (n - 1) * (2 if fills else 1) + (1 if fills else 0)
+        if need > len(self.alloc.free):
+            raise RuntimeError("ChunkAllocator: capacity reached")
+        if chunk.full():
+            chunk = chunk.add_child(self.alloc.allocate())
+            self.tails[seq_idx] = chunk
+        pairs, targets = [], [None] * n
+        if n > 1:
+            node = chunk.parent
+            while node is not None:
+                node.n_seqs += n - 1
+                node = node.parent
+            distance = chunk.parent.children.index(chunk) + 1
+            for i in range(1, n):
+                copy = self._copy_of_tail(chunk)
+                pairs.append((chunk.slot, copy.slot))
+                targets[i] = (copy.slot, copy.n_tokens)
+                copy.append_tokens(tokens, i, i + 1)
+                chunk.parent.children.insert(distance, copy)
+                copy.parent = chunk.parent
+                distance += 1
+                tail = copy
+                if copy.full():
+                    tail = copy.add_child(self.alloc.allocate())
+                self.tails.insert(seq_idx + i, tail)
+        targets[0] = (chunk.slot, chunk.n_tokens)
+        chunk.append_tokens(tokens, 0, 1)
+        if chunk.full():
+            self.tails[seq_idx] = chunk.add_child(self.alloc.allocate())
+        self.valid = False
+        return pairs, targets
 
     # attention.cpp:342-372: pre-order walk with an explicit stack, so the children of a
     # node are visited in REVERSE order; the root itself is not listed; empty chunks are.

@@ -330,3 +330,53 @@ def test_many_short_private_runs_one_item_per_wave():
     attn.ctx.set_schedule(0)
     assert_close(attn.forward(to_dev(q)), want)
     assert attn.ctx.plan_info().stream_per_wave == 1
+
+
+def test_beam_search_operations_through_the_c_abi():
+    """duplicate and append_completion (reference attention.cpp:227-261, 287-313) on the GPU cache:
+    every sequence's attention equals textbook attention over its own K/V history."""
+    rng = np.random.default_rng(21)
+    H, c = 4, 32
+    attn = make_attention(H, c, 64)
+    hist = []                                   # per sequence: (k rows, v rows) as numpy
+
+    def rows(n):
+        return (rng.standard_normal((n, H, 128)).astype(np.float16), rng.standard_normal((n, H, 128)).astype(np.float16))
+
+    k0, v0 = rows(70)                            # two full chunks and a tail of 6
+    attn.add_seq(list(range(70)), to_dev(k0), to_dev(v0))
+    k1, v1 = rows(31)
+    attn.add_seq(list(range(64)) + list(range(1000, 1031)), to_dev(np.concatenate([k0[:64], k1])),
+                 to_dev(np.concatenate([v0[:64], v1])))
+    hist = [(k0, v0), (np.concatenate([k0[:64], k1]), np.concatenate([v0[:64], v1]))]
+
+    def check():
+        n = len(hist)
+        q = rng.standard_normal((n, H, 128)).astype(np.float16)
+        out = attn.forward(to_dev(q)).float().cpu().numpy()
+        for s, (k, v) in enumerate(hist):
+            sc = np.einsum("hd,thd->ht", q[s].astype(np.float64), k.astype(np.float64)) / np.sqrt(128.0)
+            p = np.exp(sc - sc.max(axis=1, keepdims=True))
+            want = np.einsum("ht,thd->hd", p / p.sum(axis=1, keepdims=True), v.astype(np.float64))
+            np.testing.assert_allclose(out[s], want, atol=ATOL, rtol=RTOL)
+
+    check()
+    attn.duplicate(1, 2)                         # sequences 1, 2, 3 are the same now
+    hist[2:2] = [hist[1], hist[1]]
+    assert attn.tree.n_seqs == 4
+    check()
+    # beam step on sequence 2: three candidates; its tail holds 31 of 32 rows, so all three fill up
+    nk, nv = rows(3)
+    assert attn.append_completion(2, [7, 8, 9], to_dev(nk), to_dev(nv)) == 2
+    base = hist[2]
+    hist[2:3] = [(np.concatenate([base[0], nk[i:i + 1]]), np.concatenate([base[1], nv[i:i + 1]])) for i in range(3)]
+    assert attn.tree.n_seqs == 6
+    check()
+    # and the decode loop goes on from there
+    ak, av = rows(6)
+    attn.append_token(list(range(500, 506)), to_dev(ak), to_dev(av))
+    hist = [(np.concatenate([k, ak[i:i + 1]]), np.concatenate([v, av[i:i + 1]])) for i, (k, v) in enumerate(hist)]
+    check()
+    attn.remove_seq(3)
+    del hist[3]
+    check()

@@ -200,3 +200,104 @@ def test_random_histories_keep_invariants(seed):
             del model[i]
         check_invariants(t)
         assert [t.seq_tokens(i) for i in range(len(model))] == model
+
+
+# ---- beam-search operations (reference attention.cpp:227-261, 287-313; the reference's own
+# ---- test_duplicate is skipped, so these are pinned by hand-worked trees, the token-list model
+# ---- and the tree invariants) ------------------------------------------------------------------
+
+def test_duplicate_hand_worked():
+    t = PrefixTree(2, 64)
+    t.add_seq([1, 2, 3])          # root -> [1,2] -> [3]
+    t.add_seq([1, 2, 4, 5])       # [1,2] -> [4,5] -> []
+    pairs = t.duplicate(0, 2)     # two more copies of sequence 0, right after it
+    #   root(4) -> [1,2](4) -> { [3](1), [3](1), [3](1), [4,5](1) -> [](1) }
+    assert t.structure() == (4, (), [(4, (1, 2), [(1, (3,), []), (1, (3,), []), (1, (3,), []),
+                                                  (1, (4, 5), [(1, (), [])])])])
+    assert [t.seq_tokens(i) for i in range(4)] == [[1, 2, 3]] * 3 + [[1, 2, 4, 5]]
+    src = t.tails[0].slot
+    assert pairs == [(src, t.tails[1].slot), (src, t.tails[2].slot)]
+    assert len({c.slot for c in t.tails}) == 4
+    assert t.duplicate(1, 0) == [] and t.n_seqs == 4
+    check_invariants(t)
+
+
+def test_append_completion_hand_worked():
+    t = PrefixTree(2, 64)
+    t.add_seq([1, 2, 3])
+    t.add_seq([1, 2, 4, 5])
+    # three candidates for sequence 0; its tail [3] has one free row, so every candidate fills
+    # its chunk and gets an empty child at once
+    pairs, targets = t.append_completion(0, [7, 8, 9])
+    assert t.structure() == (4, (), [(4, (1, 2), [(1, (3, 7), [(1, (), [])]), (1, (3, 8), [(1, (), [])]),
+                                                  (1, (3, 9), [(1, (), [])]), (1, (4, 5), [(1, (), [])])])])
+    assert [t.seq_tokens(i) for i in range(4)] == [[1, 2, 3, 7], [1, 2, 3, 8], [1, 2, 3, 9], [1, 2, 4, 5]]
+    first = t.tails[0].parent
+    assert targets[0] == (first.slot, 1)                     # row 1 of the chunk that held [3]
+    assert [p[0] for p in pairs] == [first.slot, first.slot]
+    assert targets[1:] == [(p[1], 1) for p in pairs]
+    # a full tail without a child (append_token leaves it so) first gets its empty child
+    t2 = PrefixTree(2, 64)
+    t2.add_seq([1])
+    t2.append_token([2])
+    assert t2.tails[0].full() and not t2.tails[0].children
+    _, tg = t2.append_completion(0, [5, 6])
+    assert [t2.seq_tokens(i) for i in range(2)] == [[1, 2, 5], [1, 2, 6]]
+    assert tg[0][1] == 0 and tg[1][1] == 0
+    check_invariants(t2)
+    # a single candidate is an append to one sequence only
+    t2.append_completion(1, [9])
+    assert [t2.seq_tokens(i) for i in range(2)] == [[1, 2, 5], [1, 2, 6, 9]]
+    check_invariants(t2)
+
+
+def test_beam_operations_capacity():
+    t = PrefixTree(2, 3)
+    t.add_seq([1, 2, 3])                     # uses 2 chunks
+    before = t.structure()
+    with pytest.raises(RuntimeError, match="capacity reached"):
+        t.append_completion(0, [4, 5])       # would need 3 more chunks
+    assert t.structure() == before           # nothing changed
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_histories_with_beam_operations(seed):
+    rng = random.Random(500 + seed)
+    c = rng.choice([2, 3, 4])
+    t = PrefixTree(c, 8192)
+    model = []
+    for _ in range(150):
+        op = rng.random()
+        if op < 0.3 or not model:
+            toks = [rng.randint(0, 2) for _ in range(rng.randint(1, 10))]
+            idx, _ = t.add_seq(toks)
+            model.insert(idx, list(toks))
+        elif op < 0.5:
+            new = [rng.randint(0, 2) for _ in model]
+            t.append_token(new)
+            for m, x in zip(model, new):
+                m.append(x)
+        elif op < 0.65:
+            i, n = rng.randrange(len(model)), rng.randint(0, 3)
+            pairs = t.duplicate(i, n)
+            assert len(pairs) == n
+            for k in range(n):
+                model.insert(i + 1 + k, list(model[i]))
+        elif op < 0.85:
+            i = rng.randrange(len(model))
+            cand = [rng.randint(0, 2) for _ in range(rng.randint(1, 4))]
+            pairs, targets = t.append_completion(i, cand)
+            assert len(pairs) == len(cand) - 1 and len(targets) == len(cand)
+            base = model[i]
+            for k in range(1, len(cand)):
+                model.insert(i + k, base + [cand[k]])
+            model[i] = base + [cand[0]]
+            for k, (slot, row) in enumerate(targets):     # the row named is where the token sits
+                node = t.tails[i + k] if t.tails[i + k].n_tokens else t.tails[i + k].parent
+                assert (node.slot, node.n_tokens - 1) == (slot, row) and node.tokens[-1] == cand[k]
+        else:
+            i = rng.randrange(len(model))
+            t.remove_seq(i)
+            del model[i]
+        check_invariants(t)
+        assert [t.seq_tokens(i) for i in range(len(model))] == model

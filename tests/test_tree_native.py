@@ -138,3 +138,57 @@ def test_benchmark_trees(cfg, frac, want):
     shared = rows[(rows[:, 3] - rows[:, 2]) > 1]
     assert (len(rows), len(shared), int((shared[:, 3] - shared[:, 2]).sum())) == want
     assert int((rows[:, 1] == 0).sum()) == w.n_seqs      # one empty tail per sequence
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_histories_with_beam_operations_match_oracle(seed):
+    """duplicate / append_completion of the native manager against the restatement of reference
+    attention.cpp:227-261, 287-313: same tree, same slots, same copy pairs and row targets."""
+    rng = random.Random(900 + seed)
+    c = rng.choice([2, 3, 4, 8])
+    nat, ora = capi.Tree(c, 4096), PrefixTree(c, 4096)
+    n = 0
+    for _ in range(150):
+        op = rng.random()
+        if op < 0.3 or n == 0:
+            toks = [rng.randint(0, 2) for _ in range(rng.randint(1, 3 * c + 2))]
+            i1, _, _ = nat.add_seq(toks)
+            i2, _ = ora.add_seq(toks)
+            assert i1 == i2
+            n += 1
+        elif op < 0.5:
+            new = [rng.randint(0, 2) for _ in range(n)]
+            assert nat.append_token(new) == len(ora.append_token(new))
+        elif op < 0.65:
+            i, k = rng.randrange(n), rng.randint(0, 3)
+            assert nat.duplicate(i, k) == ora.duplicate(i, k)
+            n += k
+        elif op < 0.85:
+            i = rng.randrange(n)
+            cand = [rng.randint(0, 2) for _ in range(rng.randint(1, 4))]
+            p1, t1 = nat.append_completion(i, cand)
+            p2, t2 = ora.append_completion(i, cand)
+            assert p1 == p2 and t1 == t2
+            n += len(cand) - 1
+        else:
+            i = rng.randrange(n)
+            nat.remove_seq(i)
+            ora.remove_seq(i)
+            n -= 1
+        same_state(nat, ora)
+
+
+def test_beam_operation_errors():
+    t = capi.Tree(2, 3)
+    t.add_seq([1, 2, 3])
+    rows = t.get_chunks().copy()
+    with pytest.raises(capi.ChunkAttnError, match="capacity reached"):
+        t.append_completion(0, [4, 5])
+    with pytest.raises(capi.ChunkAttnError, match="capacity reached"):
+        t.duplicate(0, 2)
+    np.testing.assert_array_equal(t.get_chunks(), rows)     # failed calls leave the tree alone
+    with pytest.raises(capi.ChunkAttnError):
+        t.duplicate(5, 1)
+    with pytest.raises(capi.ChunkAttnError):
+        t.append_completion(-1, [1])
+    assert t.duplicate(0, 0) == [] and t.append_completion(0, []) == ([], [])
