@@ -166,6 +166,17 @@ def side_costs(attn, w, torch, capi):
     e1.record()
     torch.cuda.synchronize()
     scatter_us = e0.elapsed_time(e1) * 1e3 / reps
+    # one beam-search step on that sequence: four candidates = three tail-chunk copies and four
+    # K/V rows (wall clock with a device sync; the three new sequences are removed again)
+    k4 = torch.zeros((4, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    for rep in range(2):            # the first step loads torch's row-copy kernels: timed is the second
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        attn.append_completion(idx, [-5 - 4 * rep, -6 - 4 * rep, -7 - 4 * rep, -8 - 4 * rep], k4, k4)
+        torch.cuda.synchronize()
+        beam_us = (time.perf_counter() - t0) * 1e6
+        for i in (3, 2, 1):
+            attn.remove_seq(idx + i)
     attn.remove_seq(idx)
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
@@ -207,7 +218,7 @@ def side_costs(attn, w, torch, capi):
     norm["rotary_embedding_GBps"] = round(4 * TN * hidden * 2 / us / 1e3, 1)
     return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
-            "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
+            "beam_step_4_candidates_us": round(beam_us, 1), "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
             "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
 

@@ -74,6 +74,8 @@ SIGNATURES = {
     "ca_scatter_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "ca_put_kv_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, c_i32_p,
+                                      ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
     "ca_ctx_set_schedule": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
@@ -450,6 +452,12 @@ class KernelContext:
         arr, ptr = _i32(slots)
         _check(self._lib.ca_scatter_kv(self._h, k_ptr, v_ptr, n_tokens, tok_begin, ptr, len(slots), stream))
 
+    def put_kv_rows(self, k_ptr: int, v_ptr: int, targets: Sequence[Tuple[int, int]], stream: int = 0) -> None:
+        """Row i of k/v to row targets[i][1] of chunk targets[i][0]."""
+        flat = [x for t in targets for x in t]
+        arr, ptr = _i32(flat)
+        _check(self._lib.ca_put_kv_rows(self._h, k_ptr, v_ptr, len(targets), ptr, stream))
+
     def copy_chunk(self, src_slot: int, dst_slot: int, stream: int = 0) -> None:
         _check(self._lib.ca_copy_chunk(self._h, src_slot, dst_slot, stream))
 
@@ -639,10 +647,7 @@ class Attention:
         pairs, targets = self.tree.append_completion(seq_idx, tokens)
         for src, dst in pairs:
             self.ctx.copy_chunk(src, dst, self._stream())
-        kp, vp = self.pool_views()
-        for i, (slot, row) in enumerate(targets):       # same stream: after the copies
-            kp[slot, :, row].copy_(k[i])
-            vp[slot, :, row].copy_(v[i])
+        self.ctx.put_kv_rows(k.data_ptr(), v.data_ptr(), targets, self._stream())   # same stream: after the copies
         self.ctx.invalidate()
         return seq_idx
 

@@ -206,14 +206,12 @@ int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::T
     c10::DeviceGuard guard(t_options_.device());
     for (const auto& [src, dst] : pairs) check(ca_copy_chunk(ctx_, src, dst, stream()));
     // row i of k/v is the new token of sequence seq_idx + i (same stream: after the copies)
-    const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
-    auto chunk_view = [&](torch::Tensor& storage, int slot) {
-        return storage.narrow(0, chunk_elems * slot, chunk_elems).view({ n_heads_, chunk_size_, d_head_ });
-    };
-    for (int i = 0; i < n; i++) {
-        chunk_view(key_storage_, rows[i].slot).select(1, rows[i].row).copy_(k[i]);
-        chunk_view(value_storage_, rows[i].slot).select(1, rows[i].row).copy_(v[i]);
+    std::vector<int32_t> slot_row;
+    for (const auto& r : rows) {
+        slot_row.push_back(r.slot);
+        slot_row.push_back(r.row);
     }
+    check(ca_put_kv_rows(ctx_, k.data_ptr(), v.data_ptr(), n, slot_row.data(), stream()));
     ca_ctx_invalidate(ctx_);  // sequence lengths changed under the device tables
     return seq_idx;
 }

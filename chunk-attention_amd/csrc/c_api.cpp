@@ -613,6 +613,20 @@ int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
     return CA_OK;
 }
 
+int ca_put_kv_rows(ca_ctx* c, const void* k, const void* v, int n_rows, const int32_t* slot_row, void* stream) {
+    if (!c || n_rows < 0) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_rows == 0) return CA_OK;
+    if (!k || !v || !slot_row) return fail(CA_ERR_INVALID, "null pointer");
+    for (int i = 0; i < n_rows; i++) {
+        if (slot_row[2 * i] < 0 || slot_row[2 * i] >= c->max_chunks || slot_row[2 * i + 1] < 0 ||
+            slot_row[2 * i + 1] >= c->C) {
+            return fail(CA_ERR_INVALID, "target " + std::to_string(i) + " is outside the pool or the chunk");
+        }
+    }
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    return launch_rc(ca::launch_put_rows(a, k, v, slot_row, n_rows, static_cast<hipStream_t>(stream)), "row write launch");
+}
+
 int ca_ctx_set_plan(ca_ctx* c, int shared_seg_chunks, int stream_chunks) {
     if (!c || shared_seg_chunks < 0 || stream_chunks < 0) return fail(CA_ERR_INVALID, "bad argument");
     c->seg_chunks = shared_seg_chunks;

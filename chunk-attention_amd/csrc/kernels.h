@@ -48,6 +48,9 @@ int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32
                   const int32_t* tail_fill, int n_seqs, hipStream_t st);
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,
                    const int32_t* slots, int n_slots, hipStream_t st);
+// rows i < n of k/v ([n, H, d]) to row slot_row[2i+1] of chunk slot_row[2i] (host array)
+int launch_put_rows(const LaunchArgs& a, const void* k, const void* v, const int32_t* slot_row, int n,
+                    hipStream_t st);
 
 // Rotary position embedding (fp16).  cos_sin_cache is [max_position, rot_dim]: rot_dim/2 cosines
 // then rot_dim/2 sines per position; positions outside the cache are clamped into it.

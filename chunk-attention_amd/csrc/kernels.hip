@@ -1087,6 +1087,27 @@ __global__ __launch_bounds__(WG) void scatter_kernel(const T* __restrict__ k, co
     vpool[dst] = v[src];
 }
 
+// K/V rows to explicit places: row i of k and v goes to row targets.row[i] of chunk
+// targets.slot[i] (the beam-search step's row writes, one launch for all candidates).
+constexpr int PUT_ROWS = 64;
+struct PutTargets {
+    int32_t slot[PUT_ROWS];
+    int32_t row[PUT_ROWS];
+};
+template <typename T>
+__global__ __launch_bounds__(WG) void put_rows_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                                      T* __restrict__ kpool, T* __restrict__ vpool,
+                                                      PutTargets targets, int first, int n, int H, int C,
+                                                      int pieces) {
+    const int idx = blockIdx.x * WG + threadIdx.x;
+    if (idx >= n * H * pieces) return;
+    const int piece = idx % pieces, ih = idx / pieces, h = ih % H, i = ih / H;
+    const size_t dst = ((size_t(targets.slot[i]) * H + h) * C + targets.row[i]) * pieces + piece;
+    const size_t src = (size_t(first + i) * H + h) * pieces + piece;
+    kpool[dst] = k[src];
+    vpool[dst] = v[src];
+}
+
 }  // namespace
 
 // ---- launchers -----------------------------------------------------------------------------
@@ -1206,6 +1227,33 @@ int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_toke
                                dim3(WG), 0, st, static_cast<const uint16_t*>(k),
                                static_cast<const uint16_t*>(v), static_cast<uint16_t*>(kp),
                                static_cast<uint16_t*>(vp), args, t0, n_copy, a.H, a.C, pieces);
+        }
+        CA_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int launch_put_rows(const LaunchArgs& a, const void* k, const void* v, const int32_t* slot_row, int n,
+                    hipStream_t st) {
+    void* kp = const_cast<void*>(a.kpool);
+    void* vp = const_cast<void*>(a.vpool);
+    for (int i0 = 0; i0 < n; i0 += PUT_ROWS) {
+        const int m = (n - i0 < PUT_ROWS) ? (n - i0) : PUT_ROWS;
+        PutTargets t;
+        for (int i = 0; i < PUT_ROWS; i++) {
+            t.slot[i] = (i < m) ? slot_row[2 * (i0 + i)] : 0;
+            t.row[i] = (i < m) ? slot_row[2 * (i0 + i) + 1] : 0;
+        }
+        if (a.d % 8 == 0) {
+            const int pieces = a.d / 8, total = m * a.H * pieces;
+            hipLaunchKernelGGL(put_rows_kernel<uint4>, dim3((total + WG - 1) / WG), dim3(WG), 0, st,
+                               static_cast<const uint4*>(k), static_cast<const uint4*>(v), static_cast<uint4*>(kp),
+                               static_cast<uint4*>(vp), t, i0, m, a.H, a.C, pieces);
+        } else {
+            const int pieces = a.d, total = m * a.H * pieces;
+            hipLaunchKernelGGL(put_rows_kernel<uint16_t>, dim3((total + WG - 1) / WG), dim3(WG), 0, st,
+                               static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v),
+                               static_cast<uint16_t*>(kp), static_cast<uint16_t*>(vp), t, i0, m, a.H, a.C, pieces);
         }
         CA_LAUNCH_CHECK();
     }

@@ -140,6 +140,13 @@ int ca_scatter_kv(ca_ctx* ctx, const void* k, const void* v, int n_tokens, int t
 /* Device copy of one chunk's K and V (reference Chunk::deep_copy, chunk.cpp:93-107). */
 int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
 
+/* K/V rows to explicit places, one launch: row i of k and v ([n_rows, n_heads, d_head] on the
+ * device) goes to row slot_row[2i+1] of chunk slot_row[2i] (host array).  The device half of the
+ * row appends in reference Attention::append_completion (attention.cpp:243,253 ->
+ * Chunk::append_tokens, chunk.cpp:63-72: one tensor slice assignment per candidate and pool). */
+int ca_put_kv_rows(ca_ctx* ctx, const void* k, const void* v, int n_rows, const int32_t* slot_row,
+                   void* stream);
+
 /* Work-list shaping.  0 = choose from the device's compute-unit count and the step's size.
  * shared_seg_chunks = 1 gives one partial row set per shared chunk, the granularity of the
  * reference's partial buffers.  A work item never holds more than 64 chunks: larger values are

@@ -107,3 +107,24 @@ def test_copy_in_and_chunk_copy_beyond_4_gib():
     ctx.copy_chunk(N_SLOTS - 1, FIRST_HIGH + 40, stream)
     torch.cuda.synchronize()
     assert torch.equal(kp[FIRST_HIGH + 40], kp[N_SLOTS - 1]) and torch.equal(vp[FIRST_HIGH + 40], vp[N_SLOTS - 1])
+
+
+def test_row_writes_beyond_4_gib_and_bad_targets():
+    rng = np.random.default_rng(8)
+    kp = torch.empty((N_SLOTS, H, C, D), dtype=torch.float16, device=dev())
+    vp = torch.empty_like(kp)
+    ctx = capi.KernelContext(H, D, C, kp.data_ptr(), vp.data_ptr(), N_SLOTS)
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 70                                             # more than one launch's worth of targets
+    k = rng.standard_normal((n, H, D)).astype(np.float16)
+    v = rng.standard_normal((n, H, D)).astype(np.float16)
+    targets = [(int(FIRST_HIGH + 3 * i), int((5 * i) % C)) for i in range(n)]
+    tk, tv = to_dev(k), to_dev(v)
+    ctx.put_kv_rows(tk.data_ptr(), tv.data_ptr(), targets, stream)
+    torch.cuda.synchronize()
+    for i, (slot, row) in enumerate(targets):
+        assert np.array_equal(kp[slot, :, row].cpu().numpy(), k[i])
+        assert np.array_equal(vp[slot, :, row].cpu().numpy(), v[i])
+    for bad in [(N_SLOTS, 0), (-1, 0), (5, C), (5, -1)]:
+        with pytest.raises(capi.ChunkAttnError, match="outside the pool or the chunk"):
+            ctx.put_kv_rows(tk.data_ptr(), tv.data_ptr(), [bad], stream)
