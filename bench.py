@@ -284,6 +284,7 @@ def main() -> int:
     ap.add_argument("--no-paged", action="store_true", help="skip the private-copies baseline")
     ap.add_argument("--seg-chunks", type=int, default=0)
     ap.add_argument("--stream-chunks", type=int, default=0)
+    ap.add_argument("--stream-hint", type=int, default=0, help="non-temporal loads of private chunks: 0 by working-set size (default), 1 always, 2 never")
     ap.add_argument("--schedule", type=int, default=0, help="0 producer launch + merge launch (default), 1 single launch with in-kernel merge")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
@@ -317,6 +318,7 @@ def main() -> int:
     if args.seg_chunks or args.stream_chunks:
         attn.ctx.set_plan(args.seg_chunks, args.stream_chunks)
     attn.ctx.set_schedule(args.schedule)
+    attn.ctx.set_stream_hint(args.stream_hint)
     q_np = w.q(args.seed)
     q = torch.from_numpy(q_np).to("cuda:0")
     out = torch.empty_like(q)

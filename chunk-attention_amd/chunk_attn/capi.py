@@ -78,6 +78,7 @@ SIGNATURES = {
                                       ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
     "ca_ctx_set_schedule": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_ctx_set_stream_hint": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_read_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
@@ -463,6 +464,10 @@ class KernelContext:
 
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
+
+    def set_stream_hint(self, mode: int) -> None:
+        """Non-temporal loads of private chunks: 0 by working-set size (default), 1 always, 2 never."""
+        _check(self._lib.ca_ctx_set_stream_hint(self._h, int(mode)))
 
     def set_schedule(self, mode: int) -> None:
         """0: producer launch + merge launch (default); 1: single launch, last finisher merges."""

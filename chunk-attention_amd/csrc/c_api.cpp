@@ -94,6 +94,7 @@ struct ca_ctx {
            off_tail_slot = 0, off_tail_fill = 0;
     int schedule = 0;  // 0: partial-producing launch + merge launch; 1: one launch, last finisher merges
     int plan_schedule = 0;  // schedule the current plan was built for
+    int stream_hint = 0;    // non-temporal loads of private chunks: 0 by working-set size, 1 always, 2 never
 
     float* part = nullptr;
     size_t part_cap = 0;  // bytes
@@ -144,7 +145,11 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     // its K/V there again on the next step, and plain loads top out near 6.3 TB/s against
     // 7.2 TB/s for loads with the non-temporal hint (measured with a bare read kernel): stream
     // the private chunks around the cache then.  Smaller working sets keep plain loads.
-    a.stream_nt = (int64_t(c->plan.stream_tokens) + c->plan.shared_tokens) * 4 * c->H * c->d > (int64_t(256) << 20);
+    // The caller may know better (ca_ctx_set_stream_hint): the layers of a model each have a cache
+    // of their own and together never fit.
+    a.stream_nt = c->stream_hint == 1 ||
+                  (c->stream_hint == 0 &&
+                   (int64_t(c->plan.stream_tokens) + c->plan.shared_tokens) * 4 * c->H * c->d > (int64_t(256) << 20));
     return a;
 }
 
@@ -632,6 +637,12 @@ int ca_ctx_set_plan(ca_ctx* c, int shared_seg_chunks, int stream_chunks) {
     c->seg_chunks = shared_seg_chunks;
     c->stream_chunks = stream_chunks;
     c->valid = false;
+    return CA_OK;
+}
+
+int ca_ctx_set_stream_hint(ca_ctx* c, int mode) {
+    if (!c || mode < 0 || mode > 2) return fail(CA_ERR_INVALID, "stream hint must be 0, 1 or 2");
+    c->stream_hint = mode;
     return CA_OK;
 }
 

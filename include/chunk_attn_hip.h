@@ -153,6 +153,14 @@ int ca_put_kv_rows(ca_ctx* ctx, const void* k, const void* v, int n_rows, const 
  * cut down to that (63 for stream_chunks, whose last item may take one chunk more). */
 int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
 
+/* How the private (per-sequence) chunks are read.  0 (default): with the non-temporal hint when
+ * one forward attends more K/V than the 256 MiB last-level cache holds, plainly otherwise (a
+ * caller that repeats forwards over a small cache finds part of it there again).  1: always with
+ * the hint -- for a model whose layers each own a cache, so that nothing attended is still cached
+ * when its layer comes round again.  2: never.  Results do not depend on it.  No counterpart in
+ * the reference (its kernels use plain loads, kernel_cuda.cu:885-1086). */
+int ca_ctx_set_stream_hint(ca_ctx* ctx, int mode);
+
 /* How ca_attention is launched.  0 (default): one launch in which chunk-first and sequence-
  * first workgroups run side by side and write partial rows, then a merge launch.  1: a single
  * launch in which the workgroup that finishes the last partial of a (sequence, head) merges

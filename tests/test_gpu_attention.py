@@ -380,3 +380,18 @@ def test_beam_search_operations_through_the_c_abi():
     attn.remove_seq(3)
     del hist[3]
     check()
+
+
+def test_stream_hint_does_not_change_results():
+    """ca_ctx_set_stream_hint only picks the load instruction for private chunks."""
+    w = synth.two_level_workload("hint", groups=2, per_group=3, chunk_size=64, root=128, mid=64, unique=150, n_heads=4)
+    attn, _ = load_workload(w, 5)
+    q = to_dev(w.q(5))
+    outs = []
+    for mode in (0, 1, 2):
+        attn.ctx.set_stream_hint(mode)
+        outs.append(attn.forward(q))
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert_close(outs[0], oracle_output(attn, w.q(5), exact=True))
+    with pytest.raises(capi.ChunkAttnError, match="stream hint"):
+        attn.ctx.set_stream_hint(3)
