@@ -53,9 +53,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Partial rows are written by one workgroup and read by another, possibly on a different XCD
-// whose L2 is not coherent with the writer's.  They are therefore moved with device-scope
-// relaxed atomics (write-through stores, L2-bypassing loads): no cache-wide fence is needed,
-// only "stores done" (a workgroup barrier) before the completion counter is bumped.
+// whose L2 is not coherent with the writer's.  When both happen in one launch (single-launch
+// schedule) they are therefore moved with device-scope relaxed atomics (write-through stores,
+// L2-bypassing loads): no cache-wide fence is needed, only "stores done" (a workgroup barrier)
+// before the completion counter is bumped.
 // Before a workgroup announces its partial rows through the completion counter, every wave
 // waits until its own stores have been acknowledged: a workgroup barrier alone orders waves
 // but does not wait for their outstanding global stores.
@@ -63,13 +64,24 @@ __device__ __forceinline__ void wait_own_stores() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0)
 }
-__device__ __forceinline__ void part_store(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// coherent = the rows are read during this launch (single-launch schedule).  When a later launch
+// reads them, ordinary stores do: the end of the launch makes them visible, and they leave the L2
+// as whole lines instead of being written through 8 bytes at a time.
+__device__ __forceinline__ void part_store(float* p, float v, bool coherent) {
+    if (coherent) {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *p = v;
+    }
 }
-__device__ __forceinline__ void part_store2(float* p, float a, float b) {
-    union { f2 f; uint64_t u; } x;
-    x.f = f2{ a, b };
-    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void part_store2(float* p, float a, float b, bool coherent) {
+    if (coherent) {
+        union { f2 f; uint64_t u; } x;
+        x.f = f2{ a, b };
+        __hip_atomic_store(reinterpret_cast<uint64_t*>(p), x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *reinterpret_cast<f2*>(p) = f2{ a, b };
+    }
 }
 __device__ __forceinline__ float part_load(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -298,6 +310,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     const int32_t* __restrict__ slots = A.slots;
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
+    const bool coh = A.fuse_merge != 0;  // partial rows are read during this launch
     // A wave works on 64-token sub-tiles: one chunk at chunk size 64, half a chunk at 128, two
     // consecutive chunks of the item at 32 (their loads go out together, so a wave has the same
     // 32 KiB in flight at every chunk size).
@@ -494,8 +507,8 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
             } else {
                 float* own_row = A.part + (size_t(own) * H + h) * PART_STRIDE;
 #pragma unroll
-                for (int e = 0; e < 8; e += 2) part_store2(own_row + 4 + 8 * j + e, acc[e], acc[e + 1]);
-                if (j == 0) part_store2(own_row, m_run, l_wave);
+                for (int e = 0; e < 8; e += 2) part_store2(own_row + 4 + 8 * j + e, acc[e], acc[e + 1], coh);
+                if (j == 0) part_store2(own_row, m_run, l_wave, coh);
             }
         }
         return;
@@ -532,8 +545,8 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
         return;
     }
     float* own_row = A.part + (size_t(own) * H + h) * PART_STRIDE;
-    if (tid < D) part_store(own_row + 4 + tid, o);
-    if (tid == 0) part_store2(own_row, m, lsum);
+    if (tid < D) part_store(own_row + 4 + tid, o, coh);
+    if (tid == 0) part_store2(own_row, m, lsum, coh);
     if (!A.fuse_merge) return;
 
     // publish, count, and let whoever arrives last merge from memory
@@ -575,6 +588,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     const int32_t* __restrict__ slots = A.slots;
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
+    const bool coh = A.fuse_merge != 0;  // partial rows are read during this launch
     const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
     const int l = tid & 63, g = l >> 4, i = l & 15;
@@ -738,8 +752,8 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
         const int row = idx / (D / 4), c4 = idx % (D / 4);
         float* dst = A.part + (size_t(sm.row[row]) * H + h) * PART_STRIDE + 4 + 4 * c4;
         const f4 v = *reinterpret_cast<const f4*>(&sm.o[row * OPITCH + 4 * c4]);
-        part_store2(dst, v[0], v[1]);
-        part_store2(dst + 2, v[2], v[3]);
+        part_store2(dst, v[0], v[1], coh);
+        part_store2(dst + 2, v[2], v[3], coh);
     }
     if (w == 0 && g == 0) {
 #pragma unroll
@@ -749,7 +763,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
                 float lsum = 0.f;
 #pragma unroll
                 for (int k = 0; k < NW; k++) lsum += sm.l[k][row];
-                part_store2(A.part + (size_t(sm.row[row]) * H + h) * PART_STRIDE, m_all[mb], lsum);
+                part_store2(A.part + (size_t(sm.row[row]) * H + h) * PART_STRIDE, m_all[mb], lsum, coh);
             }
         }
     }
@@ -795,6 +809,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
     const int32_t* __restrict__ slots = A.slots;
     const int H = A.H;
     const float scale_log2 = A.scale_log2;
+    const bool coh = A.fuse_merge != 0;  // partial rows are read during this launch
     const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, known uniform
     const int l = tid & 63, g = l >> 4, i = l & 15;
@@ -972,11 +987,11 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
         const int row = row_base + mb * 16 + i;
         if (row < it.n_rows) {
             float* dst = A.part + (size_t(A.part_ptr[it.seq_begin + row] + it.part_row) * H + h) * PART_STRIDE;
-            if (g == 0) part_store2(dst, m_run[mb], l_lane[mb]);
+            if (g == 0) part_store2(dst, m_run[mb], l_lane[mb], coh);
 #pragma unroll
             for (int db = 0; db < 8; db++) {
-                part_store2(dst + 4 + 16 * db + 4 * g, oacc[mb][db][0], oacc[mb][db][1]);
-                part_store2(dst + 4 + 16 * db + 4 * g + 2, oacc[mb][db][2], oacc[mb][db][3]);
+                part_store2(dst + 4 + 16 * db + 4 * g, oacc[mb][db][0], oacc[mb][db][1], coh);
+                part_store2(dst + 4 + 16 * db + 4 * g + 2, oacc[mb][db][2], oacc[mb][db][3], coh);
             }
         }
     }
