@@ -1018,8 +1018,33 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
 // grid = (n_shared_items + n_stream_items) * H workgroups, shared items first: they have the
 // longest dependent chains and are sized to about one per compute unit, so they are done long
 // before the streaming is and the merge falls to stream workgroups, one row each.
+// What a workgroup needs before its first loads can go out comes as the leading scalar
+// arguments: with kernel-argument preload they arrive in scalar registers with the wave (the
+// first 14 dwords), so the work item's header is requested at once instead of after a round trip to the
+// argument buffer; a struct passed by value is never preloaded.  The rest is wanted later.
+struct DecodeRest {
+    const int32_t* slots;
+    half_t* out;
+    float* part;
+    const int32_t* part_ptr;
+    int32_t* counters;
+};
+constexpr int kFlagFuseMerge = 1, kFlagPerWave = 2, kFlagStreamNt = 4;
+
 template <int C>
-__global__ __launch_bounds__(WG, 2) void decode_kernel(const DecodeArgs A) {
+__global__ __launch_bounds__(WG, 2) void decode_kernel(const WorkItem* stream_items, const WorkItem* shared_items,
+                                                       const half_t* kpool, const half_t* vpool, const half_t* q,
+                                                       int n_shared_wgs, int H, int delta_tokens, int flags,
+                                                       float scale_log2, int n_stream_items, const DecodeRest rest) {
+    DecodeArgs A;
+    A.q = q; A.kpool = kpool; A.vpool = vpool; A.out = rest.out; A.part = rest.part;
+    A.shared_items = shared_items; A.stream_items = stream_items; A.slots = rest.slots;
+    A.part_ptr = rest.part_ptr; A.counters = rest.counters; A.n_shared_wgs = n_shared_wgs;
+    A.delta_tokens = delta_tokens; A.H = H; A.scale_log2 = scale_log2;
+    A.fuse_merge = (flags & kFlagFuseMerge) ? 1 : 0;
+    A.n_stream_items = n_stream_items;
+    A.stream_per_wave = (flags & kFlagPerWave) ? 1 : 0;
+    A.stream_nt = (flags & kFlagStreamNt) ? 1 : 0;
     __shared__ DecodeLds lds;
     const int bid = blockIdx.x;
     if (bid < A.n_shared_wgs) {
@@ -1168,12 +1193,20 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     d.n_stream_items = n_stream_items;
     d.stream_per_wave = a.stream_per_wave ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
+    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters };
+    const int flags = (d.fuse_merge ? kFlagFuseMerge : 0) | (d.stream_per_wave ? kFlagPerWave : 0) |
+                      (d.stream_nt ? kFlagStreamNt : 0);
+#define CA_DECODE_LAUNCH(CS)                                                                              \
+    hipLaunchKernelGGL(decode_kernel<CS>, grid, block, 0, st, d.stream_items, d.shared_items, d.kpool,   \
+                       d.vpool, d.q, d.n_shared_wgs, d.H, d.delta_tokens, flags, d.scale_log2,           \
+                       d.n_stream_items, rest)
     switch (a.C) {
-        case 32: hipLaunchKernelGGL(decode_kernel<32>, grid, block, 0, st, d); break;
-        case 64: hipLaunchKernelGGL(decode_kernel<64>, grid, block, 0, st, d); break;
-        case 128: hipLaunchKernelGGL(decode_kernel<128>, grid, block, 0, st, d); break;
+        case 32: CA_DECODE_LAUNCH(32); break;
+        case 64: CA_DECODE_LAUNCH(64); break;
+        case 128: CA_DECODE_LAUNCH(128); break;
         default: return -1;
     }
+#undef CA_DECODE_LAUNCH
     CA_LAUNCH_CHECK();
     return 0;
 }
