@@ -166,3 +166,32 @@ def test_items_never_hold_more_than_64_chunks(partition, seg, strm):
     for items in (plan["shared_items"], plan["stream_items"]):
         if len(items):
             assert items[:, 3].min() >= 1 and items[:, 3].max() <= 64
+
+
+def test_stream_items_taper_over_the_last_sequences():
+    """With the default item size, the last sequences (one fill of the device's workgroup slots,
+    or a quarter of the sequences if that is more, at most half) get items of half the length:
+    the launch drains through them.  An explicit item size switches the taper off, and sizes
+    that cannot be halved (half an item would leave waves without a tile) stay as they are."""
+    w = synth.baseline_config(1)                      # 32 sequences, 8 private chunks of 64 (+ empty tail) each
+    t = PrefixTree(w.chunk_size, 2048)
+    for s in range(w.n_seqs):
+        t.add_seq(w.tokens(s))
+    rows = rows_np(t)
+    plan = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0)["plan"]
+    check_plan(rows, t.n_seqs, w.chunk_size, plan, 1, 0)
+    per_seq = np.bincount(plan["stream_items"][:, 0], minlength=w.n_seqs)
+    # 256 compute units x 2 slots / 32 heads = 16 sequences per fill = half of the 32: the cap
+    assert per_seq[:16].tolist() == [1] * 16 and per_seq[16:].tolist() == [2] * 16
+    assert plan["stream_items"][:16, 3].tolist() == [9] * 16            # 8 chunks and the tail riding along
+    assert sorted(set(plan["stream_items"][16:, 3].tolist())) == [4, 5]
+    small = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0, n_heads=32, n_cus=64)["plan"]   # 4 per fill
+    assert np.bincount(small["stream_items"][:, 0], minlength=w.n_seqs).tolist() == [1] * 24 + [2] * 8   # a quarter
+    fixed = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0, 0, 8)["plan"]
+    assert np.bincount(fixed["stream_items"][:, 0], minlength=w.n_seqs).tolist() == [1] * 32
+    # chunk size 128: the default item is four chunks, one per wave: no taper
+    t2 = PrefixTree(128, 2048)
+    for s in range(16):
+        t2.add_seq(list(range(256)) + [10 ** 6 * (s + 1) + i for i in range(8 * 128)])
+    p2 = capi.build_tables(rows_np(t2), 16, 128, 1, 0)["plan"]
+    assert len(set(np.bincount(p2["stream_items"][:, 0], minlength=16).tolist())) == 1
