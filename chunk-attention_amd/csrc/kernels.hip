@@ -12,7 +12,7 @@
 //                   output: the second launch of a forward.  (In the single-launch schedule the
 //                   decode workgroup that completes the last partial of a (sequence, head) does
 //                   this merge itself.)
-//   append_kernel / scatter_kernel   K/V row writes into the chunk pool.
+//   append_kernel / scatter_kernel / put_rows_kernel   K/V row writes into the chunk pool.
 //
 // Partial rows live in base-2 units: max holds score*log2(e)/sqrt(d), sums and acc are
 // relative to 2^max.  Row layout: [0] max, [1] sum, [4..131] acc (fp32); rows are 640 B apart so
