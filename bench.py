@@ -83,6 +83,33 @@ def measured_traffic(workload, info):
     return int(e["decode_kernel_bytes"]), e.get("how", "")
 
 
+def cold_forward_us(attn, q, out, torch, reps=20):
+    """The forward when nothing it attends is still cached: a read of 1 GiB of other memory (four
+    times the last-level cache; a read, so that no dirty lines are left to write back) runs in
+    front of every timed forward, HIP events on the launch stream around the forward alone.  What
+    a model with many layers sees; the benchmark protocol repeats one forward."""
+    stream = torch.cuda.current_stream().cuda_stream
+    flush = torch.zeros(1 << 27, dtype=torch.int64, device="cuda:0")
+    res = {}
+    for name, hint in (("default_policy", 0), ("non_temporal_forced", 1)):
+        attn.ctx.set_stream_hint(hint)
+        attn.refresh_kernel_context()
+        total = 0.0
+        for i in range(reps + 2):
+            flush.sum()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], 0, stream)
+            e1.record()
+            e1.synchronize()
+            if i >= 2:
+                total += e0.elapsed_time(e1)
+        res[name + "_us"] = round(total * 1e3 / reps, 2)
+    attn.ctx.set_stream_hint(0)
+    del flush
+    return res
+
+
 def decode_launch_us(attn, q, out, steps, torch):
     """Average duration of the decode launch: a back-to-back train of that launch alone between
     two HIP events on the launch stream (events around every single launch add 2-3 us each)."""
@@ -370,6 +397,8 @@ def main() -> int:
                      "bytes_per_launch": decode_bytes, "avg_launch_us": round(decode_ms * 1e3, 2)},
     }
 
+    if args.stream_hint == 0:
+        result["cold_cache_forward"] = cold_forward_us(attn, q, out, torch)
     result["per_step_side_costs"] = side_costs(attn, w, torch, capi)
     if args.config == 3:
         # the two-level configuration's 32 decode steps: as given (tails never fill) and with

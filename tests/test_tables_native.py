@@ -195,3 +195,30 @@ def test_stream_items_taper_over_the_last_sequences():
         t2.add_seq(list(range(256)) + [10 ** 6 * (s + 1) + i for i in range(8 * 128)])
     p2 = capi.build_tables(rows_np(t2), 16, 128, 1, 0)["plan"]
     assert len(set(np.bincount(p2["stream_items"][:, 0], minlength=16).tolist())) == 1
+
+
+def test_shared_runs_of_different_widths_get_segments_of_similar_cost():
+    """Two-level workload: the root run (64 sequences, two 32-row items per segment, 16 chunks)
+    costs more per tile than the eight group runs (8 sequences, 8 chunks each), which are the
+    majority of the chunk-first workgroups; the root is cut into three segments instead of two so
+    that no chunk-first workgroup outlasts the others by much.  Single-run workloads keep their
+    segmentation, and an explicit segment length switches the balancing off."""
+    w = synth.baseline_config(3)
+    t = PrefixTree(w.chunk_size, 2048)
+    for s in range(w.n_seqs):
+        t.add_seq(w.tokens(s))
+    rows = rows_np(t)
+    plan = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0)["plan"]
+    check_plan(rows, t.n_seqs, w.chunk_size, plan, 1, 0)
+    items = plan["shared_items"]
+    root = items[items[:, 1] == 32]                    # 32-row items: the root run, two per segment
+    mid = items[items[:, 1] == 8]
+    assert len(root) == 6 and sorted(root[:, 3].tolist()) == [5, 5, 5, 5, 6, 6]
+    assert len(mid) == 8 and set(mid[:, 3].tolist()) == {8}
+    fixed = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0, 8, 0)["plan"]["shared_items"]
+    assert len(fixed[fixed[:, 1] == 32]) == 4
+    w2 = synth.baseline_config(1)                      # one shared run: nothing to balance against
+    t2 = PrefixTree(w2.chunk_size, 2048)
+    for s in range(w2.n_seqs):
+        t2.add_seq(w2.tokens(s))
+    assert len(capi.build_tables(rows_np(t2), t2.n_seqs, w2.chunk_size, 1, 0)["plan"]["shared_items"]) == 2
