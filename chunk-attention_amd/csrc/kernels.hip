@@ -791,15 +791,18 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
 
 // ---------------------------------------------------------------------------------------
 // wide_path: chunk-first for chunks shared by many sequences.  An item covers up to 128
-// sequences; wave w owns rows 32w .. 32w+31 (Q^T and the output accumulators stay in its
-// registers for the whole segment) and attends every token.  The segment is walked in 64-token
+// sequences; wave w owns rows 32w .. 32w+31, or 16w .. 16w+15 when the item has at most 64 (MBW
+// = 16-row blocks per wave; Q^T and the output accumulators stay in the wave's registers for the
+// whole segment), and attends every token.  The segment is walked in 64-token
 // tiles: all 256 threads stage the K and V tile in LDS once (the next tile is already on its way
 // in registers), then each wave runs the same MFMA scheme as shared_path with K operands read
 // from LDS.  Every K/V byte is fetched once per 128 sequences and no cross-wave merge is needed.
 // ---------------------------------------------------------------------------------------
-template <int C>
+template <int C, int MBW>
 __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                           int h, WidePathLds& sm) {
+    static_assert(MBW == 1 || MBW == 2, "one or two 16-row blocks per wave");
+    constexpr int MB = MBW;  // shadows the file-level constant inside this function
     WorkItem it;
     it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
     it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
@@ -815,7 +818,7 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
     const int l = tid & 63, g = l >> 4, i = l & 15;
     const int slotv = preload_slots(gi, it.slot_first, it.n_chunks, slots, l);
     const int len = it.len0 + A.delta_tokens;
-    const int row_base = 32 * w;                    // first item row of this wave
+    const int row_base = 16 * MB * w;               // first item row of this wave
     const bool active = row_base < it.n_rows;       // wave has sequences (uniform per wave)
 
     h8 qreg[MB][4];
@@ -973,8 +976,10 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int db = 0; db < 8; db++) {
-                oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[0], oacc[0][db], 0, 0, 0);
-                oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[1], oacc[1][db], 0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    oacc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[mb], oacc[mb][db], 0, 0, 0);
+                }
             }
         }
     }
@@ -1050,7 +1055,12 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const WorkItem* stream_it
     if (bid < A.n_shared_wgs) {
         const WorkItem* gi = A.shared_items + bid / A.H;
         if (gi->flags & kItemWide) {
-            wide_path<C>(A, gi, bid % A.H, lds.wd);
+            // up to 64 sequences: 16 rows per wave keep all four waves busy
+            if (gi->n_rows <= 64) {
+                wide_path<C, 1>(A, gi, bid % A.H, lds.wd);
+            } else {
+                wide_path<C, 2>(A, gi, bid % A.H, lds.wd);
+            }
         } else {
             shared_path<C>(A, gi, bid % A.H, lds.sh);
         }

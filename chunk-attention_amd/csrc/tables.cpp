@@ -103,6 +103,17 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         runs.push_back({ i, j - i });
         i = j;
     }
+    // Which runs take the row-split wide form.  From kWideMin sequences on it always pays: each
+    // K/V byte is fetched once per 128 sequences instead of once per 32.  Between kWideMinLong and
+    // kWideMin it replaces two or three 32-row workgroups per segment by one whose tiles take
+    // longer (~2 us against ~1.4 us), which halves the slot time the run takes from the streaming
+    // but lengthens its chain: worth it on long runs only (measured with 64 sequences: a 64-chunk
+    // run 28.4 -> 26.6 us per forward, a 48-chunk run 175.4 -> 168.9 us, 32- and 16-chunk runs
+    // under long private parts unchanged, the 16-chunk root of a two-level tree 37.2 -> 38.6 us).
+    auto run_wide = [&](const Run& run) {
+        const int n = rows[run.first_row].seq_end - rows[run.first_row].seq_begin;
+        return n >= kWideMin || (n >= kWideMinLong && int64_t(run.count) * chunk_size >= kWideLongTokens);
+    };
     // Segment length.  A shared workgroup may run for a good part of the step's expected
     // duration (bytes at ~6.4 TB/s) but must not outlast it.  Long segments mean fewer
     // workgroups (each pays its start-up and final merge once), fewer partial rows to write and
@@ -122,15 +133,14 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             const int n = rows[run.first_row].seq_end - rows[run.first_row].seq_begin;
             const int seg = std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
             const int n_segs = std::max({ 1, (run.count + seg / 2) / seg, ceil_div(run.count, kMaxItemChunks) });
-            wgs += int64_t(n_segs) * ceil_div(n, n >= kWideMin ? kWideRows : kMaxRows) * std::max(params.n_heads, 1);
+            wgs += int64_t(n_segs) * ceil_div(n, run_wide(run) ? kWideRows : kMaxRows) * std::max(params.n_heads, 1);
         }
         return wgs;
     };
     int base_tiles = std::max(static_cast<int>(0.3 * step_us), 4);
     while (base_tiles < 32 && shared_wgs_with(base_tiles) > int64_t(2) * params.n_cus) base_tiles++;
-    auto seg_chunks_for = [&](int n_covered) {
+    auto seg_chunks_for = [&](bool wide) {
         if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
-        const bool wide = n_covered >= kWideMin;
         const int n_tiles = std::min(base_tiles, wide ? 64 : 32);  // 64-token tiles
         return std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
     };
@@ -139,8 +149,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     // segments per run: nearest, not ceiling; but never more chunks in a segment than an item holds
     std::vector<int> run_segs(runs.size());
     for (size_t r = 0; r < runs.size(); r++) {
-        const int n = rows[runs[r].first_row].seq_end - rows[runs[r].first_row].seq_begin;
-        const int seg = seg_chunks_for(n);
+        const int seg = seg_chunks_for(run_wide(runs[r]));
         run_segs[r] = std::max({ 1, (runs[r].count + seg / 2) / seg, ceil_div(runs[r].count, kMaxItemChunks) });
     }
     // Runs of different widths (a root shared by everyone, groups below it): a tile costs more
@@ -152,14 +161,14 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     if (params.shared_seg_chunks <= 0 && runs.size() > 1) {
         auto run_cost = [&](size_t r) {
             const int n = rows[runs[r].first_row].seq_end - rows[runs[r].first_row].seq_begin;
-            const double per_tile = n >= kWideMin ? 2.0 : (n > 16 ? 1.4 : 1.0);
+            const double per_tile = run_wide(runs[r]) ? 2.0 : (n > 16 ? 1.4 : 1.0);
             return per_tile * runs[r].count * chunk_size / 64.0;
         };
         std::vector<std::pair<double, int64_t>> seg_cost;  // (cost of one segment, workgroups per head)
         int64_t total_weight = 0;
         for (size_t r = 0; r < runs.size(); r++) {
             const int n = rows[runs[r].first_row].seq_end - rows[runs[r].first_row].seq_begin;
-            const int64_t wgs = int64_t(run_segs[r]) * ceil_div(n, n >= kWideMin ? kWideRows : kMaxRows);
+            const int64_t wgs = int64_t(run_segs[r]) * ceil_div(n, run_wide(runs[r]) ? kWideRows : kMaxRows);
             seg_cost.emplace_back(run_cost(r) / run_segs[r], wgs);
             total_weight += wgs;
         }
@@ -202,7 +211,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 }
                 n_parts[r0.seq_begin + s]++;
             }
-            const bool wide = n >= kWideMin;
+            const bool wide = run_wide(run);
             const int tile_rows = wide ? kWideRows : kMaxRows;
             for (int m0 = 0; m0 < n; m0 += tile_rows) {
                 WorkItem it{};

@@ -100,6 +100,30 @@ def test_any_number_of_sharing_sequences(n_shared_seqs):
     assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
 
 
+@pytest.mark.parametrize("schedule", [0, 1])
+@pytest.mark.parametrize("n_seqs", [64, 70, 95])
+def test_long_shared_run_under_64_to_95_sequences(n_seqs, schedule):
+    # a run of 3072 tokens or more shared by 64..95 sequences is attended in the row-split wide
+    # form: one workgroup for all rows, 16 rows per wave up to 64 sequences, 32 beyond
+    w = synth.prefix_workload("long-run", n_seqs, 64, 3136, 70, n_heads=2)
+    attn, order = load_workload(w)
+    assert order == list(range(w.n_seqs))
+    attn.ctx.set_schedule(schedule)
+    attn.refresh_kernel_context()
+    info = attn.ctx.plan_info()
+    rows = attn.get_chunks()
+    plan = capi.build_tables(rows, w.n_seqs, 64, 1, 0, n_heads=2)["plan"]
+    assert len(plan["shared_items"]) == info.n_shared_items
+    assert set(plan["shared_items"][:, 7].tolist()) == {1} and plan["shared_items"][:, 1].max() == n_seqs
+    q = w.q()
+    want = oracle_output(attn, q)
+    for _ in range(2):
+        assert_close(attn.forward(to_dev(q)), want)
+    k, v = w.append_kv(0)
+    attn.append_token(w.append_tokens(0), to_dev(k), to_dev(v))
+    assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
+
+
 def test_two_level_tree_and_remove():
     w = synth.two_level_workload("two-level", 3, 5, 32, 96, 64, 40, n_heads=4)
     attn, order = load_workload(w)

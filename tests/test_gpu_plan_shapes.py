@@ -21,7 +21,7 @@ def build(c, rng):
     root = list(range(3 * c))                                         # shared by everyone
     rk, rv = rng.standard_normal((len(root), H, 128)).astype(np.float16), rng.standard_normal((len(root), H, 128)).astype(np.float16)
     n = 0
-    for g, n_in_group in enumerate((100, 9, 1)):                       # a wide group, a narrow one, a loner
+    for g, n_in_group in enumerate((100, 9, 1, 68)):                   # a wide group, a narrow one, a loner, a mid-sized one
         mid = [10 ** 4 * (g + 1) + i for i in range(2 * c)]
         mk, mv = rng.standard_normal((len(mid), H, 128)).astype(np.float16), rng.standard_normal((len(mid), H, 128)).astype(np.float16)
         for s in range(n_in_group):
