@@ -100,19 +100,19 @@ def test_any_number_of_sharing_sequences(n_shared_seqs):
     assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
 
 
-@pytest.mark.parametrize("schedule", [0, 1])
-@pytest.mark.parametrize("n_seqs", [64, 70, 95])
-def test_long_shared_run_under_64_to_95_sequences(n_seqs, schedule):
+@pytest.mark.parametrize("n_seqs,c,schedule", [(64, 64, 0), (70, 64, 0), (95, 64, 0), (64, 64, 1), (70, 64, 1),
+                                               (95, 64, 1), (64, 32, 0), (80, 32, 1), (64, 128, 0), (80, 128, 1)])
+def test_long_shared_run_under_64_to_95_sequences(n_seqs, c, schedule):
     # a run of 3072 tokens or more shared by 64..95 sequences is attended in the row-split wide
     # form: one workgroup for all rows, 16 rows per wave up to 64 sequences, 32 beyond
-    w = synth.prefix_workload("long-run", n_seqs, 64, 3136, 70, n_heads=2)
+    w = synth.prefix_workload("long-run", n_seqs, c, 3136, 70, n_heads=2)
     attn, order = load_workload(w)
     assert order == list(range(w.n_seqs))
     attn.ctx.set_schedule(schedule)
     attn.refresh_kernel_context()
     info = attn.ctx.plan_info()
     rows = attn.get_chunks()
-    plan = capi.build_tables(rows, w.n_seqs, 64, 1, 0, n_heads=2)["plan"]
+    plan = capi.build_tables(rows, w.n_seqs, c, 1, 0, n_heads=2)["plan"]
     assert len(plan["shared_items"]) == info.n_shared_items
     assert set(plan["shared_items"][:, 7].tolist()) == {1} and plan["shared_items"][:, 1].max() == n_seqs
     q = w.q()
