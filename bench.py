@@ -110,11 +110,12 @@ def cold_forward_us(attn, q, out, torch, reps=20):
     return res
 
 
-def decode_launch_us(attn, q, out, steps, torch):
-    """Average duration of the decode launch: a back-to-back train of that launch alone between
-    two HIP events on the launch stream (events around every single launch add 2-3 us each)."""
+def decode_launch_us(attn, q, out, steps, torch, mode=3):
+    """Average duration of the decode launch (mode 3), or of its sequence-first workgroups alone
+    (mode 4): a back-to-back train of that launch between two HIP events on the launch stream
+    (events around every single launch add 2-3 us each)."""
     stream = torch.cuda.current_stream().cuda_stream
-    attn.ctx.set_timing(3)
+    attn.ctx.set_timing(mode)
     for _ in range(5):
         attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], 0, stream)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -365,6 +366,8 @@ def main() -> int:
     decode_bytes = stream_bytes + shared_bytes + qo_bytes // 2
     achieved = decode_bytes / (decode_ms * 1e-3) / 1e9 if decode_ms > 0 else 0.0
     traffic, traffic_note = measured_traffic(w.name, info)
+    stream_us = decode_launch_us(attn, q, out, min(args.steps, 200), torch, mode=4) if info.n_stream_items else 0.0
+    train_gbps = stream_bytes / (stream_us * 1e-6) / 1e9 if stream_us > 0 else 0.0
     stream_gbps = stream_bytes / (ph["stream_ms"] * 1e-3) / 1e9 if ph["stream_ms"] > 0 else 0.0
 
     result = {
@@ -389,7 +392,12 @@ def main() -> int:
         "step_frac_of_hbm_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "split_phases_us": {k.replace("_ms", ""): round(v * 1e3, 2) for k, v in ph.items()},
         "unique_kv_streaming": {"GBps": round(stream_gbps, 1), "frac_of_hbm_peak": round(stream_gbps / HBM_PEAK_GBPS, 4),
-                                "bytes": stream_bytes, "note": "sequence-first phase launched alone, HIP events"},
+                                "bytes": stream_bytes, "launch_train_us": round(stream_us, 2),
+                                "launch_train_GBps": round(train_gbps, 1),
+                                "note": "sequence-first phase launched alone.  GBps: HIP events around every single launch "
+                                        "(split_phases_us.stream; the events add 2-3 us).  launch_train: a back-to-back train "
+                                        "of the launch between two events (consecutive launches overlap tail and ramp a "
+                                        "little).  The launch's duration in the committed rocprofv3 kernel trace lies between."},
         "launches_us": {"decode_kernel": round(decode_ms * 1e3, 2), "merge_kernel": round(merge_ms * 1e3, 2)},
         "roofline": {"bound": "hbm", "kernel": "decode_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,

@@ -474,7 +474,8 @@ class KernelContext:
         _check(self._lib.ca_ctx_set_schedule(self._h, int(mode)))
 
     def set_timing(self, mode: int) -> None:
-        """0 off, 1 time the fused launch, 2 run and time the three phases separately."""
+        """0 off, 1 time the fused launch, 2 run and time the three phases separately, 3 / 4 issue only
+        the decode launch / only its sequence-first workgroups (for timing a train of them)."""
         _check(self._lib.ca_ctx_set_timing(self._h, int(mode)))
 
     def read_timing(self, reset: bool = True) -> dict:

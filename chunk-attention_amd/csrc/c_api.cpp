@@ -415,6 +415,10 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
             return launch_rc(ca::launch_decode(a3, static_cast<int>(c->plan.shared_items.size()),
                                                static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
         }
+        if (c->timing == 4) {
+            // measurement aid: only the sequence-first workgroups (the stream items)
+            return run_stream(c, q, out, st);
+        }
         if (int rc = collect_timing(c)) return rc;
         CA_HIP(hipEventRecord(c->ev[0], st));
         if (c->timing == 1 && c->schedule == 0) {
@@ -447,7 +451,7 @@ int ca_ctx_set_timing(ca_ctx* c, int enable) {
     if (enable && !c->ev[0]) {
         for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
     }
-    if (enable < 0 || enable > 3) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2 or 3");
+    if (enable < 0 || enable > 4) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2, 3 or 4");
     if (int rc = collect_timing(c)) return rc;
     c->timing = enable;
     return CA_OK;

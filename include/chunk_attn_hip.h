@@ -176,7 +176,9 @@ int ca_ctx_set_schedule(ca_ctx* ctx, int mode);
  * accumulators are filled; for phase analysis, slower than the normal forward.  mode 3:
  * ca_attention issues only the decode launch (no merge: sequences with more than one partial
  * get no output) and records nothing, so that a caller can time a back-to-back train of that
- * launch between two events of its own. */
+ * launch between two events of its own.  mode 4: the same for the sequence-first phase alone:
+ * ca_attention issues one launch over the stream items only (sequences whose output needs a
+ * merge get none). */
 int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
