@@ -419,3 +419,31 @@ def test_stream_hint_does_not_change_results():
     assert_close(outs[0], oracle_output(attn, w.q(5), exact=True))
     with pytest.raises(capi.ChunkAttnError, match="stream hint"):
         attn.ctx.set_stream_hint(3)
+
+
+def test_timing_modes_leave_results_alone():
+    # HIP-event timing inside the library (modes 1, 2) and the launch-only measurement aids (3, 4)
+    w = synth.prefix_workload("timing", 6, 64, 256, 200, n_heads=4)
+    attn, _ = load_workload(w)
+    q = to_dev(w.q())
+    want = attn.forward(q).clone()
+    out = torch.empty_like(q)
+    stream = torch.cuda.current_stream().cuda_stream
+    for mode in (1, 2):
+        attn.ctx.set_timing(mode)
+        attn.ctx.read_timing(reset=True)
+        for _ in range(3):
+            attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, stream)
+        t = attn.ctx.read_timing(reset=True)
+        assert t["calls"] == 3 and t["shared_ms"] > 0 and t["merge_ms"] > 0
+        if mode == 2:
+            assert t["stream_ms"] > 0
+        assert torch.equal(out, want)
+    for mode in (3, 4):   # partial work only: outputs are not complete, nothing is recorded
+        attn.ctx.set_timing(mode)
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, stream)
+        assert attn.ctx.read_timing(reset=True)["calls"] == 0
+    attn.ctx.set_timing(0)
+    assert torch.equal(attn.forward(q), want)
+    with pytest.raises(capi.ChunkAttnError):
+        attn.ctx.set_timing(5)
