@@ -121,7 +121,9 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     // unloaded: ~1.4 us for a 32-row item, ~2 us for a wide one, and up to twice that next to
     // streaming workgroups.  When the step is short but the shared work is not (everything
     // shared, little to stream), the tile count grows until the shared workgroups fit the
-    // device's slots (two per compute unit) in one go.
+    // device's slots (two per compute unit, one for wide items) in one go (measured, 64 sequences
+    // sharing all 64 chunks: 8 wide segments of 8 chunks 24.5 us per forward, 16 of 4: 26.5,
+    // 11 of 6: 26.4, 6 of 11: 26.0, 4 of 16: 31.8).
     int64_t all_tokens = 0;
     for (int i = 0; i < n_rows; i++) {
         all_tokens += int64_t(rows[i].n_tokens) * (is_shared(rows[i]) ? 1 : rows[i].seq_end - rows[i].seq_begin);
@@ -133,7 +135,10 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             const int n = rows[run.first_row].seq_end - rows[run.first_row].seq_begin;
             const int seg = std::clamp(n_tiles * 64 / chunk_size, 1, kMaxItemChunks);
             const int n_segs = std::max({ 1, (run.count + seg / 2) / seg, ceil_div(run.count, kMaxItemChunks) });
-            wgs += int64_t(n_segs) * ceil_div(n, run_wide(run) ? kWideRows : kMaxRows) * std::max(params.n_heads, 1);
+            // a wide workgroup counts for two: it keeps a compute unit's vector and matrix units
+            // busy by itself, and a second one beside it only makes both take twice as long
+            const bool wide = run_wide(run);
+            wgs += int64_t(n_segs) * ceil_div(n, wide ? kWideRows : kMaxRows) * std::max(params.n_heads, 1) * (wide ? 2 : 1);
         }
         return wgs;
     };

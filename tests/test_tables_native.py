@@ -246,3 +246,26 @@ def test_wide_form_for_64_to_95_sequences_needs_a_long_run():
     # chunk size 32: the same 3072 tokens are 96 chunks
     assert set(shared_items(64, 96, c=32)[:, 7].tolist()) == {1}
     assert set(shared_items(64, 95, c=32)[:, 7].tolist()) == {0}
+
+
+def test_all_shared_wide_runs_get_one_workgroup_per_compute_unit():
+    """Sharing sweep at fraction 1.0 (64 sequences share all 64 chunks, nothing private): the step is
+    short, so the shared run is cut until its workgroups fit the device in one go, and a wide
+    workgroup counts for two slots: 8 segments of 8 chunks x 32 heads = 256 workgroups on 256
+    compute units.  With long private parts (fraction 0.75) the run stays in one piece."""
+    def plan_for(fraction, **kw):
+        w = synth.baseline_config(2, fraction=fraction)
+        t = PrefixTree(w.chunk_size, 8192)
+        for s in range(w.n_seqs):
+            t.add_seq(w.tokens(s))
+        rows = rows_np(t)
+        plan = capi.build_tables(rows, t.n_seqs, w.chunk_size, 1, 0, **kw)["plan"]
+        check_plan(rows, t.n_seqs, w.chunk_size, plan, 1, 0)
+        return plan["shared_items"]
+    items = plan_for(1.0)
+    assert len(items) == 8 and set(items[:, 3].tolist()) == {8} and set(items[:, 7].tolist()) == {1}
+    assert set(items[:, 1].tolist()) == {64}
+    half = plan_for(1.0, n_heads=32, n_cus=128)            # half the device: twice the segment length
+    assert len(half) == 4 and set(half[:, 3].tolist()) == {16}
+    long_private = plan_for(0.75)
+    assert len(long_private) == 1 and long_private[0, 3] == 48 and long_private[0, 7] == 1
