@@ -208,19 +208,20 @@ struct DecodeArgs {
 };
 
 // Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
-// dims 2l, 2l+1.  Rows are taken eight at a time with all their loads in flight together and
-// folded with a running maximum, so a typical merge costs one memory round trip.
+// dims 2l, 2l+1.  Rows are taken NB at a time with all their loads in flight together and
+// folded with a running maximum, so a typical merge costs one memory round trip (NB = 16 in the
+// merge launch, 8 inside the decode launch, where registers are scarce).
 // COHERENT: rows may have been written during this launch by other workgroups (device-scope
 // loads); otherwise they come from an earlier launch and plain loads do.
-template <bool COHERENT>
+template <bool COHERENT, int NB = 8>
 __device__ __forceinline__ void merge_rows(const float* __restrict__ part, int p0, int p1, int h,
                                            int H, half_t* __restrict__ out_row, int l) {
     float m_run = NEG_INF, lsum = 0.f;
     f2 o = f2{ 0.f, 0.f };
-    for (int pb = p0; pb < p1; pb += 8) {
-        f2 ml[8], v[8];
+    for (int pb = p0; pb < p1; pb += NB) {
+        f2 ml[NB], v[NB];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < NB; u++) {
             ml[u] = f2{ NEG_INF, 0.f };
             v[u] = f2{ 0.f, 0.f };
             if (pb + u < p1) {
@@ -236,14 +237,14 @@ __device__ __forceinline__ void merge_rows(const float* __restrict__ part, int p
         }
         float mb = m_run;
 #pragma unroll
-        for (int u = 0; u < 8; u++) mb = fmaxf(mb, ml[u][0]);
+        for (int u = 0; u < NB; u++) mb = fmaxf(mb, ml[u][0]);
         if (mb == NEG_INF) continue;  // nothing but empty rows so far
         const float fa = (m_run == NEG_INF) ? 0.f : fast_exp2(m_run - mb);
         o *= fa;
         lsum *= fa;
         m_run = mb;
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < NB; u++) {
             const float w = (ml[u][0] == NEG_INF) ? 0.f : fast_exp2(ml[u][0] - mb);
             o += w * v[u];
             lsum += w * ml[u][1];
@@ -1087,7 +1088,7 @@ __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ par
     const int seq = sh / H, h = sh % H;
     const int p0 = part_ptr[seq], p1 = part_ptr[seq + 1];
     if (p0 == p1) return;  // written directly by a stream item
-    merge_rows<false>(part, p0, p1, h, H, out + (size_t(seq) * H + h) * D, l);
+    merge_rows<false, 16>(part, p0, p1, h, H, out + (size_t(seq) * H + h) * D, l);
 }
 
 __global__ __launch_bounds__(WG) void fill_kernel(int32_t* __restrict__ p, int n, int32_t value) {
