@@ -109,7 +109,9 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     // longer (~2 us against ~1.4 us), which halves the slot time the run takes from the streaming
     // but lengthens its chain: worth it on long runs only (measured with 64 sequences: a 64-chunk
     // run 28.4 -> 26.6 us per forward, a 48-chunk run 175.4 -> 168.9 us, 32- and 16-chunk runs
-    // under long private parts unchanged, the 16-chunk root of a two-level tree 37.2 -> 38.6 us).
+    // under long private parts unchanged, the 16-chunk root of a two-level tree 37.2 -> 38.6 us;
+    // with 48 sequences, 48 shared chunks and 1024 private tokens 133.6 -> 130.3 us, 40 sequences,
+    // 64 chunks and 512 tokens 72.0 -> 66.7 us, 56 sequences sharing all 64 chunks 27.0 -> 23.6 us).
     auto run_wide = [&](const Run& run) {
         const int n = rows[run.first_row].seq_end - rows[run.first_row].seq_begin;
         return n >= kWideMin || (n >= kWideMinLong && int64_t(run.count) * chunk_size >= kWideLongTokens);

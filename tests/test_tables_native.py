@@ -224,10 +224,11 @@ def test_shared_runs_of_different_widths_get_segments_of_similar_cost():
     assert len(capi.build_tables(rows_np(t2), t2.n_seqs, w2.chunk_size, 1, 0)["plan"]["shared_items"]) == 2
 
 
-def test_wide_form_for_64_to_95_sequences_needs_a_long_run():
+def test_wide_form_for_33_to_95_sequences_needs_a_long_run():
     """Chunks covering 96 sequences or more always take the row-split wide form (flag 1, one item
-    of up to 128 rows per segment).  From 64 to 95 sequences they take it when their run holds at
-    least 3072 tokens; shorter runs, and anything under 64 sequences, stay with 32-row items."""
+    of up to 128 rows per segment).  From 33 to 95 sequences (more than one 32-row item) they take
+    it when their run holds at least 3072 tokens; shorter runs, and anything up to 32 sequences,
+    stay with 32-row items."""
     def shared_items(n_seqs, shared_chunks, c=64):
         t = PrefixTree(c, 8192)
         prefix = list(range(shared_chunks * c))
@@ -239,7 +240,8 @@ def test_wide_form_for_64_to_95_sequences_needs_a_long_run():
         return plan["shared_items"]
 
     for n_seqs, chunks, wide in ((64, 48, True), (64, 47, False), (64, 16, False), (95, 48, True),
-                                 (63, 64, False), (96, 4, True), (130, 4, True)):
+                                 (63, 64, True), (33, 48, True), (33, 47, False), (32, 64, False),
+                                 (96, 4, True), (130, 4, True)):
         items = shared_items(n_seqs, chunks)
         assert set(items[:, 7].tolist()) == {1 if wide else 0}, (n_seqs, chunks)
         assert items[:, 1].max() == (min(n_seqs, 128) if wide else 32), (n_seqs, chunks)
