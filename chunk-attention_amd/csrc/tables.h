@@ -75,7 +75,7 @@ constexpr int kMaxRows = 32;    // sequences per shared work item (M tile)
 constexpr int kWideRows = 128;  // sequences per wide shared work item
 constexpr int kWideMin = 96;    // chunks covering at least this many sequences use wide items
 constexpr int kWideMinLong = 33;       // ... and from this many on (more than one M tile) when they belong to a long run:
-constexpr int kWideLongTokens = 3072;  // a run of at least this many tokens
+constexpr int kWideLongTokens = 2048;  // a run of at least this many tokens
 constexpr int32_t kItemWide = 1;
 
 struct Plan {

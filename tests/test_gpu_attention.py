@@ -104,7 +104,7 @@ def test_any_number_of_sharing_sequences(n_shared_seqs):
                                                (95, 64, 1), (64, 32, 0), (80, 32, 1), (64, 128, 0), (80, 128, 1),
                                                (33, 64, 0), (40, 64, 1), (49, 32, 0), (63, 128, 1)])
 def test_long_shared_run_under_33_to_95_sequences(n_seqs, c, schedule):
-    # a run of 3072 tokens or more shared by 33..95 sequences is attended in the row-split wide
+    # a run of 2048 tokens or more shared by 33..95 sequences is attended in the row-split wide
     # form: one workgroup for all rows, 16 rows per wave up to 64 sequences, 32 beyond
     w = synth.prefix_workload("long-run", n_seqs, c, 3136, 70, n_heads=2)
     attn, order = load_workload(w)

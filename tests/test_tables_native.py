@@ -227,7 +227,7 @@ def test_shared_runs_of_different_widths_get_segments_of_similar_cost():
 def test_wide_form_for_33_to_95_sequences_needs_a_long_run():
     """Chunks covering 96 sequences or more always take the row-split wide form (flag 1, one item
     of up to 128 rows per segment).  From 33 to 95 sequences (more than one 32-row item) they take
-    it when their run holds at least 3072 tokens; shorter runs, and anything up to 32 sequences,
+    it when their run holds at least 2048 tokens; shorter runs, and anything up to 32 sequences,
     stay with 32-row items."""
     def shared_items(n_seqs, shared_chunks, c=64):
         t = PrefixTree(c, 8192)
@@ -239,15 +239,15 @@ def test_wide_form_for_33_to_95_sequences_needs_a_long_run():
         check_plan(rows, t.n_seqs, c, plan, 1, 0)
         return plan["shared_items"]
 
-    for n_seqs, chunks, wide in ((64, 48, True), (64, 47, False), (64, 16, False), (95, 48, True),
-                                 (63, 64, True), (33, 48, True), (33, 47, False), (32, 64, False),
+    for n_seqs, chunks, wide in ((64, 32, True), (64, 31, False), (64, 16, False), (95, 32, True),
+                                 (63, 64, True), (33, 32, True), (33, 31, False), (32, 64, False),
                                  (96, 4, True), (130, 4, True)):
         items = shared_items(n_seqs, chunks)
         assert set(items[:, 7].tolist()) == {1 if wide else 0}, (n_seqs, chunks)
         assert items[:, 1].max() == (min(n_seqs, 128) if wide else 32), (n_seqs, chunks)
-    # chunk size 32: the same 3072 tokens are 96 chunks
-    assert set(shared_items(64, 96, c=32)[:, 7].tolist()) == {1}
-    assert set(shared_items(64, 95, c=32)[:, 7].tolist()) == {0}
+    # chunk size 32: the same 2048 tokens are 64 chunks
+    assert set(shared_items(64, 64, c=32)[:, 7].tolist()) == {1}
+    assert set(shared_items(64, 63, c=32)[:, 7].tolist()) == {0}
 
 
 def test_all_shared_wide_runs_get_one_workgroup_per_compute_unit():
