@@ -7,7 +7,8 @@
 //                   first phase (stream_path): a run of one sequence's own chunks is streamed
 //                   at HBM speed (16-byte coalesced loads, fp32 online softmax) into one
 //                   partial row, or straight into the output when nothing else is merged.
-//                   Chunks covering ~100 sequences or more take the row-split wide_path.
+//                   Chunks covering many sequences (from about 100 on, and from 33 on in long
+//                   shared runs: the work list says which) take the row-split wide_path.
 //   merge_kernel    merges the partial rows of every (sequence, head) and writes the normalised
 //                   output: the second launch of a forward.  (In the single-launch schedule the
 //                   decode workgroup that completes the last partial of a (sequence, head) does
