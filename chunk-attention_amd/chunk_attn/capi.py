@@ -51,7 +51,7 @@ SIGNATURES = {
     "ca_ctx_valid": (ctypes.c_int, [ctypes.c_void_p]),
     "ca_ctx_invalidate": (None, [ctypes.c_void_p]),
     "ca_ctx_delta_tokens": (ctypes.c_int, [ctypes.c_void_p]),
-    "ca_ctx_set_delta_tokens": (None, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_ctx_set_delta_tokens": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_attention": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                     ctypes.c_int, ctypes.c_void_p]),
     "ca_attn_chunks_first": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
@@ -429,7 +429,7 @@ class KernelContext:
 
     @delta_tokens.setter
     def delta_tokens(self, v: int) -> None:
-        self._lib.ca_ctx_set_delta_tokens(self._h, v)
+        _check(self._lib.ca_ctx_set_delta_tokens(self._h, v))
 
     def attention(self, q_ptr: int, out_ptr: int, n_seqs: int, partition: int = 0, stream: int = 0) -> None:
         _check(self._lib.ca_attention(self._h, q_ptr, out_ptr, n_seqs, partition, stream))

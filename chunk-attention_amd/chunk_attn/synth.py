@@ -48,6 +48,40 @@ def normal_fp16(seed: int, stream: int, shape: Tuple[int, ...], sigma: float = 1
     return normal(seed, stream, n, sigma).astype(np.float16).reshape(shape)
 
 
+def _signed64(x: int) -> int:
+    x &= (1 << 64) - 1
+    return x - (1 << 64) if x >= (1 << 63) else x
+
+
+def normal_fp16_torch(seed: int, stream: int, shape: Tuple[int, ...], sigma: float, device):
+    """normal_fp16 evaluated on `device` with torch: the same counters, hash and Box-Muller
+    transform (int64 arithmetic wraps like uint64; right shifts are made logical by masking),
+    so that large workloads need not be drawn on the host.  The float64 log/cos of the device
+    may differ from numpy's in the last place, which survives the rounding to fp16 for at most
+    a handful of elements per tensor: use normal_fp16 where bit-identical values matter."""
+    import torch
+
+    def mix(x):
+        x = (x ^ ((x >> 30) & ((1 << 34) - 1))) * _signed64(0xBF58476D1CE4E5B9)
+        x = (x ^ ((x >> 27) & ((1 << 37) - 1))) * _signed64(0x94D049BB133111EB)
+        return x ^ ((x >> 31) & ((1 << 33) - 1))
+
+    n = int(np.prod(shape))
+    with np.errstate(over="ignore"):
+        key = int(_mix64(np.uint64(seed) * np.uint64(0x9E3779B97F4A7C15) + np.uint64(stream)))
+    out = torch.empty(n, dtype=torch.float16, device=device)
+    step = 1 << 24   # bounded temporaries
+    for o in range(0, n, step):
+        m = min(step, n - o)
+        ctr = torch.arange(o, o + m, dtype=torch.int64, device=device)
+        bits = mix(ctr * _signed64(0xD1342543DE82EF95) + _signed64(key))
+        u1 = (((bits >> 40) & 0xFFFFFF).to(torch.float64) + 0.5) / float(1 << 24)
+        u2 = ((bits & 0xFFFFFF).to(torch.float64) + 0.5) / float(1 << 24)
+        z = torch.sqrt(-2.0 * torch.log(u1)) * torch.cos(2.0 * np.pi * u2)
+        out[o:o + m] = (z * sigma).to(torch.float32).to(torch.float16)
+    return out.reshape(shape)
+
+
 @dataclass
 class Segment:
     """A run of tokens of one sequence: ids plus the generator stream of its K and V."""
@@ -91,6 +125,22 @@ class Workload:
         ks = [draw(seg.k_stream, len(seg.ids)) for seg in self.seqs[s]]
         vs = [draw(seg.v_stream, len(seg.ids)) for seg in self.seqs[s]]
         return np.concatenate(ks, axis=0), np.concatenate(vs, axis=0)
+
+    def kv_torch(self, s: int, seed: int = 0, device="cuda:0"):
+        """kv(s) drawn on the device (see normal_fp16_torch): fp16 torch tensors [T, H, d]."""
+        import torch
+
+        def draw(stream: int, n: int):
+            if stream >= STREAM_K_UNIQUE:
+                return normal_fp16_torch(seed, stream, (n, self.n_heads, self.d_head), self.sigma, device)
+            key = ("torch", str(device), seed, stream, n)
+            if key not in self._cache:
+                self._cache[key] = normal_fp16_torch(seed, stream, (n, self.n_heads, self.d_head), self.sigma, device)
+            return self._cache[key]
+
+        ks = [draw(seg.k_stream, len(seg.ids)) for seg in self.seqs[s]]
+        vs = [draw(seg.v_stream, len(seg.ids)) for seg in self.seqs[s]]
+        return torch.cat(ks, dim=0), torch.cat(vs, dim=0)
 
     def q(self, seed: int = 0) -> np.ndarray:
         return normal_fp16(seed, STREAM_Q, (self.n_seqs, self.n_heads, self.d_head), self.sigma)

@@ -128,7 +128,7 @@ std::vector<Chunk*> Attention::append_token(const std::vector<int>& tokens, torc
         check(ca_append_kv(ctx_, k.data_ptr(), v.data_ptr(), n, stream()));
     }
     tree_->append_token_ids(tokens);
-    ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1);
+    check(ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1));
     return fresh;
 }
 
@@ -167,7 +167,7 @@ std::vector<Chunk*> Attention::append_token_rotary(const std::vector<int>& token
                                 is_neox ? 1 : 0, n, stream()));
     }
     tree_->append_token_ids(tokens);
-    ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1);
+    check(ca_ctx_set_delta_tokens(ctx_, ca_ctx_delta_tokens(ctx_) + 1));
     return fresh;
 }
 

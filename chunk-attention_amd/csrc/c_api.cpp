@@ -100,6 +100,10 @@ struct ca_ctx {
     size_t part_cap = 0;  // bytes
     int32_t* counters = nullptr;  // [n_seqs * H] partials finished per (sequence, head)
     size_t counters_cap = 0;      // bytes
+    // Device buffers that were outgrown.  Launches already queued may still read them, and
+    // hipFree waits for the whole device, so they are kept until the context is destroyed
+    // (capacities double: together they never hold more than the live buffer does).
+    std::vector<void*> retired;
 
     // optional timing: events recorded on the caller's stream around the launches.
     // 1: the fused launch; 2: forward run as three timed launches (chunk-first, sequence-first, merge)
@@ -112,13 +116,15 @@ struct ca_ctx {
 
 namespace {
 
-int ensure_dev(char** p, size_t* cap, size_t need) {
+// Makes *p hold at least `need` bytes.  Growth at least doubles the capacity and retires the old
+// buffer instead of freeing it: nothing on the decode step's path waits for the device.
+int ensure_dev(ca_ctx* c, char** p, size_t* cap, size_t need) {
     if (need <= *cap) return CA_OK;
-    if (*p) CA_HIP(hipFree(*p));
-    *p = nullptr;
-    *cap = 0;
-    const size_t want = align_up(need + need / 4, 4096);
-    CA_HIP(hipMalloc(reinterpret_cast<void**>(p), want));
+    const size_t want = align_up(std::max(need + need / 4, 2 * *cap), 4096);
+    void* fresh = nullptr;
+    CA_HIP(hipMalloc(&fresh, want));
+    if (*p) c->retired.push_back(*p);
+    *p = static_cast<char*>(fresh);
     *cap = want;
     return CA_OK;
 }
@@ -187,7 +193,7 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     c->off_tail_fill = place(p.tail_fill.size() * 4);
     const size_t total = std::max<size_t>(off, 64);
 
-    if (int rc = ensure_dev(&c->dev_blob, &c->dev_blob_cap, total)) return rc;
+    if (int rc = ensure_dev(c, &c->dev_blob, &c->dev_blob_cap, total)) return rc;
     const int hb = c->next_host;
     c->next_host ^= 1;
     // the staging buffer may still be the source of an earlier asynchronous upload
@@ -215,12 +221,12 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     CA_HIP(hipEventRecord(c->host_blob_free[hb], st));
 
     const size_t part_bytes = std::max<size_t>(size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4, 256);
-    if (int rc = ensure_dev(reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
+    if (int rc = ensure_dev(c, reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
     // completion counters (single-launch schedule only; a change of schedule rebuilds the plan and
     // comes through here): they start at zero, and each forward leaves them at zero again
     if (c->schedule != 0) {
         const int n_counters = std::max(c->n_seqs * c->H, 1);
-        if (int rc = ensure_dev(reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
+        if (int rc = ensure_dev(c, reinterpret_cast<char**>(&c->counters), &c->counters_cap, size_t(n_counters) * 4)) return rc;
         if (int rc = launch_rc(ca::launch_fill(c->counters, n_counters, 0, st), "counter reset")) return rc;
     }
     c->partition = partition;
@@ -352,6 +358,7 @@ void ca_ctx_destroy(ca_ctx* c) {
     if (c->dev_blob) (void)hipFree(c->dev_blob);
     if (c->part) (void)hipFree(c->part);
     if (c->counters) (void)hipFree(c->counters);
+    for (void* p : c->retired) (void)hipFree(p);
     for (int i = 0; i < 2; i++) {
         if (c->host_blob_free[i]) {
             (void)hipEventSynchronize(c->host_blob_free[i]);
@@ -393,8 +400,12 @@ void ca_ctx_invalidate(ca_ctx* c) {
     if (c) c->valid = false;
 }
 int ca_ctx_delta_tokens(const ca_ctx* c) { return c ? c->delta_tokens : 0; }
-void ca_ctx_set_delta_tokens(ca_ctx* c, int delta_tokens) {
-    if (c) c->delta_tokens = delta_tokens;
+int ca_ctx_set_delta_tokens(ca_ctx* c, int delta_tokens) {
+    if (!c) return fail(CA_ERR_INVALID, "null context");
+    // a negative value would put the next appended row in front of its chunk
+    if (delta_tokens < 0) return fail(CA_ERR_INVALID, "delta_tokens must not be negative");
+    c->delta_tokens = delta_tokens;
+    return CA_OK;
 }
 
 int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition, void* stream) {
@@ -448,10 +459,10 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
 
 int ca_ctx_set_timing(ca_ctx* c, int enable) {
     if (!c) return fail(CA_ERR_INVALID, "null context");
+    if (enable < 0 || enable > 4) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2, 3 or 4");
     if (enable && !c->ev[0]) {
         for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
     }
-    if (enable < 0 || enable > 4) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2, 3 or 4");
     if (int rc = collect_timing(c)) return rc;
     c->timing = enable;
     return CA_OK;
@@ -491,6 +502,7 @@ int ca_attn_seqs_first(ca_ctx* c, const void* q, void* out, int n_seqs, void* st
 int ca_append_kv(ca_ctx* c, const void* k, const void* v, int n_seqs, void* stream) {
     if (int rc = check_ready(c, k, n_seqs)) return rc;
     if (n_seqs > 0 && !v) return fail(CA_ERR_INVALID, "null device pointer");
+    if (c->delta_tokens < 0) return fail(CA_ERR_STATE, "delta_tokens is negative");
     for (int s = 0; s < n_seqs; s++) {
         if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
             return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
@@ -572,6 +584,7 @@ int ca_rope_append_kv(ca_ctx* c, const int64_t* positions, void* q, const void* 
     if (c->d % 8 != 0 || 64 % (c->d / 8) != 0) {
         return fail(CA_ERR_INVALID, "fused rotary append needs d_head in {8, 16, 32, 64, 128, 256, 512}");
     }
+    if (c->delta_tokens < 0) return fail(CA_ERR_STATE, "delta_tokens is negative");
     for (int s = 0; s < n_seqs; s++) {
         if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
             return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");

@@ -1111,7 +1111,7 @@ __global__ __launch_bounds__(WG) void append_kernel(const T* __restrict__ k, con
     if (idx >= n_seqs * H * pieces) return;
     const int piece = idx % pieces, sh = idx / pieces, h = sh % H, seq = sh / H;
     const int row = tail_fill[seq] + delta_tokens;
-    if (row >= C) return;  // host guarantees a free row; never write outside the chunk
+    if (row < 0 || row >= C) return;  // host guarantees a free row; never write outside the chunk
     const size_t dst = ((size_t(tail_slot[seq]) * H + h) * C + row) * pieces + piece;
     kpool[dst] = k[idx];
     vpool[dst] = v[idx];

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(WG) void rope_append_kernel(
     const size_t src = size_t(sh) * d + 8 * piece;
     const size_t dst = ((size_t(tail_slot[seq]) * H + h) * C + row) * d + 8 * piece;
     if (role == 2) {
-        if (row < C) *reinterpret_cast<h8*>(vpool + dst) = *reinterpret_cast<const h8*>(v + src);
+        if (row >= 0 && row < C) *reinterpret_cast<h8*>(vpool + dst) = *reinterpret_cast<const h8*>(v + src);
         return;
     }
     const half_t* in = (role == 0) ? q : k;
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(WG) void rope_append_kernel(
     }
     if (role == 0) {
         *reinterpret_cast<h8*>(q + src) = own;
-    } else if (row < C) {  // host guarantees a free row; never write outside the chunk
+    } else if (row >= 0 && row < C) {  // host guarantees a free row; never write outside the chunk
         *reinterpret_cast<h8*>(kpool + dst) = own;
     }
 }

@@ -71,7 +71,8 @@ int ca_refresh_kernel_context(ca_ctx* ctx, const ca_chunk_row* rows, int n_rows,
 int ca_ctx_valid(const ca_ctx* ctx);
 void ca_ctx_invalidate(ca_ctx* ctx);
 int ca_ctx_delta_tokens(const ca_ctx* ctx);
-void ca_ctx_set_delta_tokens(ca_ctx* ctx, int delta_tokens);
+/* delta_tokens < 0 is rejected (CA_ERR_INVALID): it would address rows in front of a chunk. */
+int ca_ctx_set_delta_tokens(ca_ctx* ctx, int delta_tokens);
 
 /* Replaces attention(ctx, q, out, partition) (kernel_cuda.cu:1320-1329).  partition 0:
  * chunks covering more than tpp_threshold sequences are attended chunk-first, the rest per

@@ -274,6 +274,48 @@ def test_forward_under_graph_capture():
         assert_close(out, oracle_output(attn, qn))
 
 
+def test_captured_forward_is_bound_to_its_delta_tokens():
+    """delta_tokens travels as a kernel argument, so a captured forward keeps the value it was
+    captured with: replayed after an append it attends the cache as it was at capture time (the
+    appended token is ignored); the eager forward sees the new token.  Callers that capture
+    re-capture after every append_token."""
+    w = synth.prefix_workload("gd", 4, 64, 128, 30, n_heads=4)
+    attn, _ = load_workload(w)
+    rng = np.random.default_rng(9)
+    qn = rand16(rng, w.n_seqs, w.n_heads, 128)
+    q = to_dev(qn)
+    out = torch.empty_like(q)
+    before = attn.forward(q).clone()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, side.cuda_stream)   # warm-up
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, torch.cuda.current_stream().cuda_stream)
+    k, v = rand16(rng, w.n_seqs, w.n_heads, 128), rand16(rng, w.n_seqs, w.n_heads, 128)
+    attn.append_token(w.append_tokens(0), to_dev(3 * k), to_dev(v))
+    assert attn.ctx.valid and attn.ctx.delta_tokens == 1      # tables untouched, only delta moved
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, before)
+    eager = attn.forward(q)
+    assert not torch.equal(eager, before)
+    assert_close(eager, oracle_output(attn, qn))
+
+
+def test_negative_delta_tokens_is_rejected():
+    w = synth.prefix_workload("nd", 2, 64, 64, 10, n_heads=2)
+    attn, _ = load_workload(w)
+    attn.refresh_kernel_context()
+    with pytest.raises(capi.ChunkAttnError) as e:
+        attn.ctx.delta_tokens = -1
+    assert e.value.code == -1 and attn.ctx.delta_tokens == 0
+    with pytest.raises(capi.ChunkAttnError):
+        attn.ctx.set_timing(7)
+
+
 @pytest.mark.parametrize("c", [32, 64, 128])
 def test_repeated_forwards_are_bit_identical(c):
     """The default schedule merges partial rows in a fixed order, so a forward is a pure function

@@ -5,7 +5,8 @@ import pytest
 import torch
 
 from chunk_attn import synth
-from gpu_helpers import assert_close, load_workload, oracle_output, to_dev
+from gpu_helpers import (assert_chunk_holds, assert_close, load_workload, oracle_output, oracle_tree_rows,
+                         textbook_on_original, to_dev)
 
 pytestmark = pytest.mark.gpu
 
@@ -15,6 +16,11 @@ def test_config_against_oracle(cfg):
     w = synth.baseline_config(cfg)
     attn, order = load_workload(w)
     assert order == list(range(w.n_seqs))
+    # independent of what the attention oracle reads back: the tree is the oracle's tree, and
+    # chunks hold the rows the workload generated (a shared one, and a private one of the last sequence)
+    np.testing.assert_array_equal(attn.get_chunks(), oracle_tree_rows(w))
+    assert_chunk_holds(attn, w, 0, 1)
+    assert_chunk_holds(attn, w, w.n_seqs - 1, w.seq_len(w.n_seqs - 1) // w.chunk_size - 1)
     q = w.q()
     qd = to_dev(q)
     out0 = attn.forward(qd)
@@ -29,6 +35,49 @@ def test_config_against_oracle(cfg):
     assert paged.ctx.plan_info().n_shared_chunks == 0
     assert_close(outp, want)
     np.testing.assert_allclose(outp.float().cpu().numpy(), out0.float().cpu().numpy(), atol=2e-3, rtol=1e-2)
+
+
+SWEEP_SAMPLES = (0, 31, 63)
+
+
+@pytest.mark.parametrize("fraction", [0.0, 0.25, 0.5, 0.75, 1.0])
+def test_config3_sharing_sweep(fraction):
+    """Batch 64, 4096 tokens of context, the given fraction of it shared (reference scenario:
+    tests/benchmark_chunk_attn.py:73-97; checks as tests/test_chunk_attn_cuda.py:19-72).  4 GiB of
+    K/V at fraction 0: drawn on the device; the sampled sequences are checked against float64
+    attention over host copies of the very tensors that were inserted."""
+    w = synth.baseline_config(2, fraction)
+    shared = int(round(4096 * fraction))
+    attn, order, kept = load_workload(w, keep=SWEEP_SAMPLES)
+    assert order == list(range(64))
+    np.testing.assert_array_equal(attn.get_chunks(), oracle_tree_rows(w))
+    q = w.q()
+    qd = to_dev(q)
+    want = {s: textbook_on_original(w, q, s, kv=kept[s]) for s in SWEEP_SAMPLES}
+    out0 = attn.forward(qd)
+    info = attn.ctx.plan_info()
+    assert info.n_shared_chunks == shared // 64 and info.shared_tokens == shared
+    assert info.stream_tokens == 64 * (4096 - shared)
+    assert (info.n_shared_items > 0) == (shared > 0)
+    for s in SWEEP_SAMPLES:
+        assert_close(out0[s], want[s])
+    assert_chunk_holds(attn, w, 0, 0, kv=kept[0])       # first chunk (shared unless fraction 0)
+    assert_chunk_holds(attn, w, 63, 63, kv=kept[63])     # last full chunk of the last sequence
+    out2 = attn.forward(qd, 2)
+    np.testing.assert_allclose(out2.float().cpu().numpy(), out0.float().cpu().numpy(), atol=2e-3, rtol=1e-2)
+    for s in SWEEP_SAMPLES:
+        assert_close(out2[s], want[s])
+    if fraction == 0.5:
+        ref = oracle_output(attn, q, partition=0)       # the reference's CPU path on the same cache
+        assert_close(out0, ref)
+        assert_close(out2, ref)
+    # private copies of the same K/V (no sharing) give the same answer
+    paged, _, _ = load_workload(synth.paged_variant(w), keep=())
+    outp = paged.forward(qd)
+    assert paged.ctx.plan_info().n_shared_chunks == 0
+    np.testing.assert_allclose(outp.float().cpu().numpy(), out0.float().cpu().numpy(), atol=2e-3, rtol=1e-2)
+    for s in SWEEP_SAMPLES:
+        assert_close(outp[s], want[s])
 
 
 def test_config4_decode_steps():
