@@ -54,6 +54,8 @@ SIGNATURES = {
     "ca_ctx_set_delta_tokens": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_attention": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                     ctypes.c_int, ctypes.c_void_p]),
+    "ca_attention_noalloc": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                            ctypes.c_void_p]),
     "ca_attn_chunks_first": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                             ctypes.c_void_p]),
     "ca_attn_seqs_first": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -433,6 +435,11 @@ class KernelContext:
 
     def attention(self, q_ptr: int, out_ptr: int, n_seqs: int, partition: int = 0, stream: int = 0) -> None:
         _check(self._lib.ca_attention(self._h, q_ptr, out_ptr, n_seqs, partition, stream))
+
+    def attention_noalloc(self, q_ptr: int, out_ptr: int, n_seqs: int, stream: int = 0) -> None:
+        """ca_attention (partition 0) with the partial rows in the library's static device scratch:
+        allocates nothing; fails when the tables need more rows than the scratch holds."""
+        _check(self._lib.ca_attention_noalloc(self._h, q_ptr, out_ptr, n_seqs, stream))
 
     def attn_chunks_first(self, q_ptr: int, n_seqs: int, stream: int = 0) -> None:
         _check(self._lib.ca_attn_chunks_first(self._h, q_ptr, n_seqs, stream))

@@ -344,6 +344,8 @@ int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k
         for (int i = 0; i < 2 && err == hipSuccess; i++) {
             err = hipEventCreateWithFlags(&c->host_blob_free[i], hipEventDisableTiming);
         }
+        // address of this device's static scratch (for ca_attention_noalloc), once per device
+        if (err == hipSuccess) err = static_cast<hipError_t>(ca::scratch_setup(c->device));
         if (err != hipSuccess) {
             ca_ctx_destroy(c);
             return fail_hip(err, "context setup");
@@ -455,6 +457,32 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
         c->ev_pending = true;
         return CA_OK;
     });
+}
+
+int ca_attention_noalloc(ca_ctx* c, const void* q, void* out, int n_seqs, void* stream) {
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
+    if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
+    if (n_seqs == 0) return CA_OK;
+    // nothing here may build or upload tables: they must already be those of the default forward
+    if (c->partition != 0 || c->schedule != 0 || c->plan_schedule != 0) {
+        return fail(CA_ERR_STATE, "the tables were built for another partition or schedule: "
+                                  "ca_attention_noalloc runs partition 0 in the two-launch schedule only");
+    }
+    float* scratch = ca::scratch_ptr(c->device);
+    if (!scratch) return fail(CA_ERR_STATE, "the static scratch of this device was not set up");
+    const size_t need = size_t(c->plan.n_part_rows) * c->H * ca::PART_STRIDE * 4;
+    if (need > ca::kScratchBytes) {
+        return fail(CA_ERR_INVALID, "this forward needs " + std::to_string(need) + " bytes of partial rows, the static "
+                                    "scratch holds " + std::to_string(ca::kScratchBytes) + ": use ca_attention");
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ca::LaunchArgs a = launch_args(c, q, out);
+    a.part = scratch;  // every row that the merge reads is written by the decode launch first
+    if (int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                             static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch")) return rc;
+    if (c->plan.n_part_rows == 0) return CA_OK;
+    return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
 }
 
 int ca_ctx_set_timing(ca_ctx* c, int enable) {

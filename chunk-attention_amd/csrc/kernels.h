@@ -36,6 +36,14 @@ struct LaunchArgs {
     bool stream_per_wave = false;
 };
 
+// Static device scratch for the entry point that allocates nothing: a file-scope __device__
+// array (kScratchBytes per GPU, held until the process ends) that stands in for the partial-row
+// buffer.  scratch_setup resolves its address on `device`, which must be the current device
+// (every GPU has its own copy at its own address); scratch_ptr returns what it found, or null.
+constexpr size_t kScratchBytes = size_t(32) << 20;
+int scratch_setup(int device);   // 0 or a positive hipError_t
+float* scratch_ptr(int device);
+
 // All return 0, -1 for an unsupported shape, or a positive hipError_t.
 // One launch over the first n_shared_items shared items and the first n_stream_items stream
 // items.  fuse_merge: the workgroup finishing the last partial of a (sequence, head) writes

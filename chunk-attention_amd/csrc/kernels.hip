@@ -1160,7 +1160,28 @@ __global__ __launch_bounds__(WG) void put_rows_kernel(const T* __restrict__ k, c
     vpool[dst] = v[src];
 }
 
+// Partial rows of the allocation-free forward.  In host code this name is only a handle for
+// hipGetSymbolAddress: the kernels get the resolved device address as an argument.
+static __device__ __align__(256) float scratch[kScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {};
+
 }  // namespace
+
+int scratch_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    g_scratch_ptr[device] = static_cast<float*>(ptr);
+    return 0;
+}
+
+float* scratch_ptr(int device) {
+    return (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+}
 
 // ---- launchers -----------------------------------------------------------------------------
 

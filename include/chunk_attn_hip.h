@@ -81,6 +81,19 @@ int ca_ctx_set_delta_tokens(ca_ctx* ctx, int delta_tokens);
 int ca_attention(ca_ctx* ctx, const void* q, void* out, int n_seqs, int partition,
                  void* stream);
 
+/* ca_attention (partition 0, default schedule) for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  It calls no hipMalloc / hipFree or other allocating routine: the partial rows go to
+ * a static device array of CA_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs
+ * on until the process ends, instead of the context's own buffer.  Fails with CA_ERR_INVALID when
+ * the forward's partial rows (n_part_rows * n_heads * 640 bytes, see ca_ctx_plan_info) exceed
+ * that, and with CA_ERR_STATE when the tables are not those of partition 0 in the default
+ * schedule (it never rebuilds them).  All contexts on one GPU share the array: calls that
+ * overlap on one GPU (different streams or threads) race; calls on one stream are safe.  Nothing
+ * in the array needs clearing between calls (every row read is written first). */
+#define CA_NOALLOC_SCRATCH_BYTES (32u << 20)
+int ca_attention_noalloc(ca_ctx* ctx, const void* q, void* out, int n_seqs, void* stream);
+
 /* Replaces attn_chunks_first(ctx, q) (kernel_cuda.cu:1118-1193): partial (max, sum, P.V)
  * of every shared segment into the context's partial buffer. */
 int ca_attn_chunks_first(ca_ctx* ctx, const void* q, int n_seqs, void* stream);
