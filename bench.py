@@ -83,15 +83,17 @@ def measured_traffic(workload, info):
     return int(e["decode_kernel_bytes"]), e.get("how", "")
 
 
-def cold_forward_us(attn, q, out, torch, reps=20):
+def cold_forward_us(attn, q, out, torch, reps=20, hints=(("default_policy", 0), ("non_temporal_forced", 1))):
     """The forward when nothing it attends is still cached: a read of 1 GiB of other memory (four
     times the last-level cache; a read, so that no dirty lines are left to write back) runs in
     front of every timed forward, HIP events on the launch stream around the forward alone.  What
-    a model with many layers sees; the benchmark protocol repeats one forward."""
+    a model with many layers sees; the benchmark protocol repeats one forward.  Also returned: the
+    decode launch alone under the same protocol (events recorded inside the library around that
+    launch, default policy)."""
     stream = torch.cuda.current_stream().cuda_stream
     flush = torch.zeros(1 << 27, dtype=torch.int64, device="cuda:0")
     res = {}
-    for name, hint in (("default_policy", 0), ("non_temporal_forced", 1)):
+    for name, hint in hints:
         attn.ctx.set_stream_hint(hint)
         attn.refresh_kernel_context()
         total = 0.0
@@ -106,8 +108,92 @@ def cold_forward_us(attn, q, out, torch, reps=20):
                 total += e0.elapsed_time(e1)
         res[name + "_us"] = round(total * 1e3 / reps, 2)
     attn.ctx.set_stream_hint(0)
+    attn.refresh_kernel_context()
+    attn.ctx.set_timing(1)
+    for i in range(reps + 2):
+        if i == 2:
+            attn.ctx.read_timing(reset=True)
+        flush.sum()
+        attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], 0, stream)
+    t = attn.ctx.read_timing(reset=True)
+    attn.ctx.set_timing(0)
+    res["decode_launch_us"] = round(t["shared_ms"] * 1e3 / max(t["calls"], 1), 2)
     del flush
     return res
+
+
+def pybind_forward_us(w, q, steps, warmup, torch, seed):
+    """The drop-in class as a caller of the reference would use it: chunk_attn.Attention.forward
+    (output allocation, validity check and both launches), same protocol as time_forward.  Returns
+    (us per forward, us per forward of the C-ABI call on the same cache with a preallocated output)."""
+    import numpy as np
+    import chunk_attn
+    attn = pybind_cache(w, torch, seed, extra_chunks_per_seq=6)
+    for _ in range(warmup):
+        out = attn.forward(q)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = attn.forward(q)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / steps
+    # table refresh through the class, host time per call (the upload is asynchronous):
+    # "tree changed" = forced rebuild (tree walk, plan, upload); "tails rolled" = what a decode
+    # step pays when last chunks fill up: reserve() + the in-place patch of the tables
+    # (three in a row at a time: the uploads come from a ring of four staging buffers, and a
+    # longer train would time the wait for the device to release one)
+    rebuild_us = 0.0
+    for _ in range(5):
+        torch.cuda.synchronize()
+        attn.forward(q)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            attn.refresh_kernel_context(True)
+        rebuild_us += (time.perf_counter() - t0) * 1e6 / 15
+    torch.cuda.synchronize()
+    kz = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    reserve_us, roll_us, n_rolled, rolls = 0.0, 0.0, 0, 0
+    c = w.chunk_size
+    for t in range(5 * c):
+        attn.append_token([1_900_000_000 - t * 4096 - s for s in range(w.n_seqs)], kz, kz)
+        if any(x.n_tokens == c for x in attn.tails):     # full last chunks: the next reserve rolls them
+            # (no device sync in front: the first launch after one costs the host 10 us more)
+            t0 = time.perf_counter()
+            fresh = attn.reserve()                       # tree work + one Python object per new chunk
+            t1 = time.perf_counter()
+            attn.refresh_kernel_context()                # the tables: patched in place, upload queued
+            t2 = time.perf_counter()
+            if rolls or t >= c:                          # the first patch is not timed
+                reserve_us += (t1 - t0) * 1e6
+                roll_us += (t2 - t1) * 1e6
+                n_rolled += len(fresh)
+            rolls += 1
+    torch.cuda.synchronize()
+    timed = max(rolls - 1, 1)
+    tables = {"tree_changed_us": round(rebuild_us, 1), "tails_rolled_us": round(roll_us / timed, 1),
+              "reserve_call_us": round(reserve_us / timed, 1),
+              "tails_rolled_per_patch": n_rolled // timed, "patches_timed": rolls - 1,
+              "note": "host time per call through chunk_attn.Attention; tree_changed = refresh_kernel_context(True): tree "
+                      "walk + tables + upload; tails_rolled = refresh_kernel_context() after reserve() gave full last "
+                      "chunks a successor: tables patched in place + upload (reserve_call_us is that reserve(), which "
+                      "also builds one Python object per new chunk)"}
+    return us, out, tables
+
+
+def pybind_cache(w, torch, seed, extra_chunks_per_seq=1):
+    """The workload in a cache of the pybind11 class."""
+    import numpy as np
+    import chunk_attn
+    need = sum(w.seq_len(s) // w.chunk_size + 1 + extra_chunks_per_seq for s in range(w.n_seqs)) + 8
+    per_chunk = w.chunk_size * w.n_heads * w.d_head * 2 * 2
+    attn = chunk_attn.Attention(n_heads=w.n_heads, d_head=w.d_head, chunk_size=w.chunk_size,
+                                memory_mb=-(-need * per_chunk // (1 << 20)), dtype=torch.float16,
+                                device=torch.device("cuda:0"))
+    for s in range(w.n_seqs):
+        k, v = w.kv(s, seed)
+        attn.add_seq(w.tokens(s), torch.from_numpy(np.ascontiguousarray(k)).to("cuda:0"),
+                     torch.from_numpy(np.ascontiguousarray(v)).to("cuda:0"))
+    return attn
 
 
 def decode_launch_us(attn, q, out, steps, torch, mode=3):
@@ -128,7 +214,7 @@ def decode_launch_us(attn, q, out, steps, torch, mode=3):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
-def side_costs(attn, w, torch, capi):
+def side_costs(attn, w, torch, capi, operators=False):
     """Per-decode-step costs outside the timed forward: a forced table rebuild (tree walk, plan,
     upload) and the append kernel, as wall-clock microseconds between device syncs."""
     import numpy as np
@@ -209,6 +295,13 @@ def side_costs(attn, w, torch, capi):
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
     copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
+    base = {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
+            "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
+            "beam_step_4_candidates_us": round(beam_us, 1), "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
+            "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
+            "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
+    if not operators:
+        return base
     # the layer's norm operators on a prefill batch of 16384 rows of H*d (128 MiB per tensor, so
     # that a launch outlasts the host's ~10 us per call; launch trains timed with events on the
     # current stream): rms_norm reads and writes the rows once, the fused form reads and writes
@@ -244,34 +337,44 @@ def side_costs(attn, w, torch, capi):
     us = e0.elapsed_time(e1) * 1e3 / reps
     norm["rotary_embedding_%dx%d_us" % (TN, hidden)] = round(us, 1)
     norm["rotary_embedding_GBps"] = round(4 * TN * hidden * 2 / us / 1e3, 1)
-    return {**norm, "table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
-            "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
-            "beam_step_4_candidates_us": round(beam_us, 1), "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
-            "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
-            "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
+    return {**norm, **base}
 
 
 def decode_loop(w, torch, capi, synth, seed, unique_tokens):
-    """The configuration's decode loop on a fresh cache: per step one append_token (K/V rows of
-    every sequence into the tails, chunk fill -> reserve -> table rebuild when a tail is full)
-    and one forward, through the torch-tensor interface; wall-clock per step."""
+    """The configuration's decode loop on a fresh cache of the pybind11 class: per step one
+    append_token (K/V rows of every sequence into the last chunks; when those are full: reserve,
+    new chunks, tables patched in place) and one forward, host work included.  us_per_step: the
+    loop free-running; per-step figures: a second pass with a device sync after every step."""
     lw = synth.two_level_workload(w.name + "-loop", 8, 8, w.chunk_size, 1024, 512, unique_tokens,
                                   n_heads=w.n_heads, append_steps=w.append_steps)
-    attn = build_cache(lw, torch, capi, seed)
-    q = torch.from_numpy(lw.q(seed)).to("cuda:0")
-    kv = [tuple(torch.from_numpy(a).to("cuda:0") for a in lw.append_kv(t, seed)) for t in range(lw.append_steps)]
-    toks = [lw.append_tokens(t) for t in range(lw.append_steps)]
-    attn.forward(q)
-    torch.cuda.synchronize()
-    new_chunks, t0 = 0, time.perf_counter()
-    for t in range(lw.append_steps):
-        new_chunks += attn.append_token(toks[t], kv[t][0], kv[t][1])
+    res = {}
+    for timed_per_step in (False, True):
+        attn = pybind_cache(lw, torch, seed, extra_chunks_per_seq=2)
+        q = torch.from_numpy(lw.q(seed)).to("cuda:0")
+        kv = [tuple(torch.from_numpy(a).to("cuda:0") for a in lw.append_kv(t, seed)) for t in range(lw.append_steps)]
+        toks = [lw.append_tokens(t) for t in range(lw.append_steps)]
         attn.forward(q)
-    torch.cuda.synchronize()
-    us = (time.perf_counter() - t0) * 1e6 / lw.append_steps
-    return {"steps": lw.append_steps, "unique_tokens_at_start": unique_tokens, "us_per_step": round(us, 1),
-            "chunks_added": int(new_chunks),
-            "note": "append_token + forward per step through the ctypes/torch interface, host work included"}
+        torch.cuda.synchronize()
+        new_chunks, per_step, t0 = [], [], time.perf_counter()
+        for t in range(lw.append_steps):
+            t1 = time.perf_counter()
+            new_chunks.append(len(attn.append_token(toks[t], kv[t][0], kv[t][1])))
+            attn.forward(q)
+            if timed_per_step:
+                torch.cuda.synchronize()
+                per_step.append((time.perf_counter() - t1) * 1e6)
+        torch.cuda.synchronize()
+        if not timed_per_step:
+            res["us_per_step"] = round((time.perf_counter() - t0) * 1e6 / lw.append_steps, 1)
+        else:
+            rolled = [i for i, n in enumerate(new_chunks) if n]
+            plain = sorted(x for i, x in enumerate(per_step) if i not in rolled and i > 0)
+            res["synced_step_median_us"] = round(plain[len(plain) // 2], 1)
+            res["synced_steps_that_added_chunks_us"] = {str(i): round(per_step[i], 1) for i in rolled}
+        del attn
+    return {"steps": lw.append_steps, "unique_tokens_at_start": unique_tokens, **res,
+            "chunks_added": int(sum(new_chunks)),
+            "note": "append_token + forward per step through chunk_attn.Attention (pybind11), host work included"}
 
 
 def cpu_baseline(attn, q_np, budget_s, torch):
@@ -310,6 +413,10 @@ def main() -> int:
     ap.add_argument("--fraction", type=float, default=0.5, help="shared fraction for configuration 2")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget, 0 to skip")
     ap.add_argument("--no-paged", action="store_true", help="skip the private-copies baseline")
+    ap.add_argument("--operators", action="store_true",
+                    help="also time the layer operators around the attention call (rms_norm, fused_add_rms_norm and "
+                         "rotary_embedding on a prefill-sized batch): outside the metric, off by default")
+    ap.add_argument("--no-pybind", action="store_true", help="skip timing the forward through the pybind11 class")
     ap.add_argument("--seg-chunks", type=int, default=0)
     ap.add_argument("--stream-chunks", type=int, default=0)
     ap.add_argument("--stream-hint", type=int, default=0, help="non-temporal loads of private chunks: 0 by working-set size (default), 1 always, 2 never")
@@ -405,9 +512,29 @@ def main() -> int:
                      "bytes_per_launch": decode_bytes, "avg_launch_us": round(decode_ms * 1e3, 2)},
     }
 
+    cold = None
     if args.stream_hint == 0:
-        result["cold_cache_forward"] = cold_forward_us(attn, q, out, torch)
-    result["per_step_side_costs"] = side_costs(attn, w, torch, capi)
+        cold = cold_forward_us(attn, q, out, torch)
+        result["cold_cache_forward"] = cold
+        # FETCH_SIZE counts L2 misses, which the 256 MiB last-level cache may serve: when the
+        # attended bytes fit it, repeated forwards are not an HBM measurement and the cold
+        # figure is the HBM fraction to quote
+        cold_gbps = decode_bytes / (cold["decode_launch_us"] * 1e-6) / 1e9
+        result["roofline"]["achieved_cold"] = round(cold_gbps, 1)
+        result["roofline"]["frac_cold"] = round(cold_gbps / HBM_PEAK_GBPS, 4)
+        result["roofline"]["cold_launch_us"] = cold["decode_launch_us"]
+        result["roofline"]["fits_last_level_cache"] = bool(stream_bytes + shared_bytes <= (256 << 20))
+        result["roofline"]["cold_note"] = ("decode launch after 1 GiB of other memory was read, HIP events recorded inside "
+                                           "the library around that launch (they add about 2 us: the fraction is a lower bound)")
+    if not args.no_pybind:
+        pyb_us, pyb_out, pyb_tables = pybind_forward_us(w, q, args.steps, args.warmup, torch, args.seed)
+        torch.cuda.synchronize()
+        result["table_refresh_pybind"] = pyb_tables
+        result["forward_pybind_us"] = round(pyb_us, 2)
+        result["forward_pybind_minus_c_abi_us"] = round(pyb_us - ms * 1e3, 2)
+        result["forward_pybind_max_abs_diff"] = float((pyb_out.float() - out.float()).abs().max())
+        del pyb_out
+    result["per_step_side_costs"] = side_costs(attn, w, torch, capi, args.operators)
     if args.config == 3:
         # the two-level configuration's 32 decode steps: as given (tails never fill) and with
         # 100 private tokens, where every tail fills at step 28 (reserve + table rebuild)
@@ -422,10 +549,18 @@ def main() -> int:
         physical = stream_bytes + shared_bytes
         torch.cuda.synchronize()
         diff = float((pout.float() - out.float()).abs().max())
+        ratio = logical / physical
         result["paged_baseline"] = {"us_per_step": round(pms * 1e3, 2), "speedup": round(pms / ms, 3),
-                                    "kv_sharing_ratio": round(logical / physical, 3),
+                                    "kv_sharing_ratio": round(ratio, 3),
+                                    "speedup_over_ratio": round(pms / ms / ratio, 3),
                                     "GBps": round((logical + qo_bytes) / (pms * 1e-3) / 1e9, 1),
                                     "max_abs_diff_vs_shared": diff}
+        if cold is not None:
+            pcold = cold_forward_us(pattn, q, pout, torch, reps=8, hints=(("default_policy", 0),))
+            result["paged_baseline"]["cold_us_per_step"] = pcold["default_policy_us"]
+            result["paged_baseline"]["cold_speedup"] = round(pcold["default_policy_us"] / cold["default_policy_us"], 3)
+            result["paged_baseline"]["cold_speedup_over_ratio"] = round(
+                pcold["default_policy_us"] / cold["default_policy_us"] / ratio, 3)
         del pattn
 
     if args.cpu_seconds > 0:

@@ -48,6 +48,7 @@ SIGNATURES = {
     "ca_ctx_destroy": (None, [ctypes.c_void_p]),
     "ca_refresh_kernel_context": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ChunkRow),
                                                  ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "ca_ctx_roll_tails": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_ctx_valid": (ctypes.c_int, [ctypes.c_void_p]),
     "ca_ctx_invalidate": (None, [ctypes.c_void_p]),
     "ca_ctx_delta_tokens": (ctypes.c_int, [ctypes.c_void_p]),
@@ -92,6 +93,9 @@ SIGNATURES = {
     "ca_ctx_read_partials_raw": (ctypes.c_int, [ctypes.c_void_p, c_f32_p, ctypes.c_int64, ctypes.c_void_p]),
     "ca_tables_build": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ChunkRow)] +
                         [ctypes.c_int] * 9),
+    "ca_tables_build_like": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
+                                            ctypes.POINTER(ChunkRow), ctypes.c_int, ctypes.c_int]),
+    "ca_tables_roll_tails": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, c_i32_p, c_i32_p, ctypes.c_int]),
     "ca_tables_destroy": (None, [ctypes.c_void_p]),
     "ca_tables_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
     "ca_tables_plan_sizes": (ctypes.c_int, [ctypes.c_void_p, c_int_p]),
@@ -106,6 +110,7 @@ SIGNATURES = {
     "ca_tree_remove_seq": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_tree_clear": (ctypes.c_int, [ctypes.c_void_p]),
     "ca_tree_reserve": (ctypes.c_int, [ctypes.c_void_p, c_int_p]),
+    "ca_tree_reserve_tails": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, c_i32_p, ctypes.c_int, c_int_p]),
     "ca_tree_append_token": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, c_int_p]),
     "ca_tree_get_chunks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ChunkRow), ctypes.c_int,
                                           c_int_p]),
@@ -191,6 +196,14 @@ class Tree:
         n = ctypes.c_int()
         _check(self._lib.ca_tree_reserve(self._h, ctypes.byref(n)))
         return n.value
+
+    def reserve_tails(self) -> Tuple[List[int], List[int]]:
+        """reserve() that reports what it added: (sequence indices, slots of their new last chunks)."""
+        cap = max(self.n_seqs, 1)
+        seqs, slots = (ctypes.c_int32 * cap)(), (ctypes.c_int32 * cap)()
+        n = ctypes.c_int()
+        _check(self._lib.ca_tree_reserve_tails(self._h, seqs, slots, cap, ctypes.byref(n)))
+        return list(seqs[: n.value]), list(slots[: n.value])
 
     def append_token(self, tokens: Sequence[int]) -> int:
         arr, ptr = _i32(tokens)
@@ -347,23 +360,43 @@ def max_chunks_for(memory_mb: int, chunk_size: int, n_heads: int, d_head: int, e
     return load().ca_tree_max_chunks_for(memory_mb, chunk_size, n_heads, d_head, elem_bytes)
 
 
-def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: int = 1,
+class HostTables:
+    """Host-only table set (ca_tables_*): the flattening ca_refresh_kernel_context performs, and
+    the patch ca_ctx_roll_tails applies, without a device."""
+
+    def __init__(self, rows: np.ndarray, n_seqs: int, chunk_size: int = 0, tpp_threshold: int = 1,
                  partition: int = 0, shared_seg_chunks: int = 0, stream_chunks: int = 0,
-                 n_heads: int = 32, n_cus: int = 256) -> dict:
-    """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
-    (work items as [n, 16] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
-    len0, flags (1 = wide shared item), 8 inline slots; an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
-    lib = load()
-    rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
-    h = ctypes.c_void_p()
-    _check(lib.ca_tables_build(ctypes.byref(h), rows.ctypes.data_as(ctypes.POINTER(ChunkRow)),
-                               rows.shape[0], n_seqs, chunk_size, tpp_threshold, partition,
-                               shared_seg_chunks, stream_chunks, n_heads, n_cus))
-    try:
+                 n_heads: int = 32, n_cus: int = 256, like: Optional["HostTables"] = None):
+        """like: build for other rows with the parameters and the work-item sizes of that table set
+        (what a patched table keeps) instead of the ones given here."""
+        self._lib = load()
+        rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
+        self._h = ctypes.c_void_p()
+        rp = rows.ctypes.data_as(ctypes.POINTER(ChunkRow))
+        if like is not None:
+            _check(self._lib.ca_tables_build_like(ctypes.byref(self._h), like._h, rp, rows.shape[0], n_seqs))
+        else:
+            _check(self._lib.ca_tables_build(ctypes.byref(self._h), rp, rows.shape[0], n_seqs, chunk_size,
+                                             tpp_threshold, partition, shared_seg_chunks, stream_chunks,
+                                             n_heads, n_cus))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h is not None and h.value:
+            self._lib.ca_tables_destroy(h)
+
+    def roll_tails(self, delta_tokens: int, seqs: Sequence[int], slots: Sequence[int]) -> None:
+        a, ap = _i32(seqs)
+        b, bp = _i32(slots)
+        _check(self._lib.ca_tables_roll_tails(self._h, delta_tokens, ap, bp, len(seqs)))
+
+    def info(self) -> PlanInfo:
         info = PlanInfo()
-        _check(lib.ca_tables_info(h, ctypes.byref(info)))
-        n_slots = ctypes.c_int()
-        _check(lib.ca_tables_plan_sizes(h, ctypes.byref(n_slots)))
+        _check(self._lib.ca_tables_info(self._h, ctypes.byref(info)))
+        return info
+
+    def ref(self) -> dict:
+        info = self.info()
         t = {
             "final_idx": np.zeros(info.n_chunks, np.int32),
             "slots": np.zeros(info.n_chunks, np.int32),
@@ -373,11 +406,17 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
             "seq_n_tokens": np.zeros(info.n_seqs, np.int32),
             "seq_chunk_map": np.zeros((info.n_seqs, info.max_seq_n_chunks), np.int32),
         }
-        _check(lib.ca_tables_ref(h, *[t[k].ctypes.data_as(c_i32_p) for k in (
+        _check(self._lib.ca_tables_ref(self._h, *[t[k].ctypes.data_as(c_i32_p) for k in (
             "final_idx", "slots", "begins", "ends", "offsets", "seq_n_tokens", "seq_chunk_map")]))
         t["n_shared"] = info.n_shared_chunks
         t["partial_rows"] = info.ref_partial_rows
         t["max_seq_n_chunks"] = info.max_seq_n_chunks
+        return t
+
+    def plan(self) -> dict:
+        info = self.info()
+        n_slots = ctypes.c_int()
+        _check(self._lib.ca_tables_plan_sizes(self._h, ctypes.byref(n_slots)))
         p = {
             "shared_items": np.zeros((info.n_shared_items, 16), np.int32),
             "stream_items": np.zeros((info.n_stream_items, 16), np.int32),
@@ -387,14 +426,24 @@ def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: 
             "tail_slot": np.zeros(info.n_seqs, np.int32),
             "tail_fill": np.zeros(info.n_seqs, np.int32),
         }
-        _check(lib.ca_tables_plan(h, *[p[k].ctypes.data_as(c_i32_p) for k in (
+        _check(self._lib.ca_tables_plan(self._h, *[p[k].ctypes.data_as(c_i32_p) for k in (
             "shared_items", "stream_items", "slots", "seq_len", "part_ptr", "tail_slot", "tail_fill")]))
         p["n_part_rows"] = info.n_part_rows
         p["shared_tokens"] = info.shared_tokens
         p["stream_tokens"] = info.stream_tokens
-        return {"ref": t, "plan": p}
-    finally:
-        lib.ca_tables_destroy(h)
+        p["stream_per_wave"] = info.stream_per_wave
+        return p
+
+
+def build_tables(rows: np.ndarray, n_seqs: int, chunk_size: int, tpp_threshold: int = 1,
+                 partition: int = 0, shared_seg_chunks: int = 0, stream_chunks: int = 0,
+                 n_heads: int = 32, n_cus: int = 256) -> dict:
+    """Host-only flattening of get_chunks rows: reference-form tables and the packed work list
+    (work items as [n, 16] int32: seq_begin, n_rows, slot_first, n_chunks, part_row, pos0,
+    len0, flags (1 = wide shared item), 8 inline slots; an item writes partial row part_ptr[seq] + part_row of each covered seq)."""
+    t = HostTables(rows, n_seqs, chunk_size, tpp_threshold, partition, shared_seg_chunks, stream_chunks,
+                   n_heads, n_cus)
+    return {"ref": t.ref(), "plan": t.plan()}
 
 
 class KernelContext:
@@ -417,6 +466,17 @@ class KernelContext:
         rows = np.ascontiguousarray(rows, np.int32).reshape(-1, 4)
         _check(self._lib.ca_refresh_kernel_context(
             self._h, rows.ctypes.data_as(ctypes.POINTER(ChunkRow)), rows.shape[0], n_seqs, stream))
+
+    def roll_tails(self, seqs: Sequence[int], slots: Sequence[int], stream: int = 0) -> bool:
+        """Patches the tables after reserve() gave the sequences `seqs` the new last chunks `slots`
+        (and folds delta_tokens in).  False when the tables cannot be patched (they are untouched)."""
+        a, ap = _i32(seqs)
+        b, bp = _i32(slots)
+        rc = self._lib.ca_ctx_roll_tails(self._h, ap, bp, len(seqs), stream)
+        if rc == -3:
+            return False
+        _check(rc)
+        return True
 
     @property
     def valid(self) -> bool:
@@ -590,10 +650,13 @@ class Attention:
         self.ctx.invalidate()
 
     def reserve(self) -> int:
-        n = self.tree.reserve()
-        if n:
-            self.ctx.invalidate()
-        return n
+        seqs, slots = self.tree.reserve_tails()
+        if seqs:
+            # full last chunks got an empty successor and nothing else changed since the tables
+            # were built: patch them; anything else is rebuilt from a tree walk at the next refresh
+            if not (self.ctx.valid and self.ctx.roll_tails(seqs, slots, self._stream())):
+                self.ctx.invalidate()
+        return len(seqs)
 
     def refresh_kernel_context(self, force: bool = False) -> None:
         if force or not self.ctx.valid:

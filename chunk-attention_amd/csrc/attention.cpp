@@ -99,11 +99,38 @@ void Attention::remove_seq(int seq_idx) { tree_->remove_seq(seq_idx); }
 
 void Attention::clear() { tree_->clear(); }
 
-std::vector<Chunk*> Attention::reserve() { return tree_->reserve(); }
+std::vector<Chunk*> Attention::reserve() { return reserve_and_note(); }
+
+std::vector<Chunk*> Attention::reserve_and_note() {
+    const uint64_t before = tree_->version();
+    std::vector<int> seqs;
+    std::vector<Chunk*> fresh = tree_->reserve(&seqs);
+    if (fresh.empty()) return fresh;
+    rolled_version_ = 0;
+    if (ca_ctx_valid(ctx_) && tables_version_ == before) {
+        // the only change since the tables were built: full last chunks got an empty successor
+        rolled_seqs_.assign(seqs.begin(), seqs.end());
+        rolled_slots_.clear();
+        for (const Chunk* c : fresh) rolled_slots_.push_back(c->slot());
+        rolled_version_ = tree_->version();
+    }
+    return fresh;
+}
 
 void Attention::refresh_kernel_context(bool force) {
     if (!force && ca_ctx_valid(ctx_) && tables_version_ == tree_->version()) return;
     c10::DeviceGuard guard(t_options_.device());
+    if (!force && rolled_version_ != 0 && rolled_version_ == tree_->version() && ca_ctx_valid(ctx_)) {
+        rolled_version_ = 0;
+        const int rc = ca_ctx_roll_tails(ctx_, rolled_seqs_.data(), rolled_slots_.data(),
+                                         static_cast<int>(rolled_seqs_.size()), stream());
+        if (rc == CA_OK) {
+            tables_version_ = tree_->version();
+            return;
+        }
+        if (rc != CA_ERR_STATE) check(rc);  // CA_ERR_STATE: not patchable, tables untouched: rebuild
+    }
+    rolled_version_ = 0;
     const auto infos = tree_->get_chunks();
     std::vector<ca_chunk_row> rows(infos.size());
     for (size_t i = 0; i < infos.size(); i++) {
@@ -121,7 +148,7 @@ std::vector<Chunk*> Attention::append_token(const std::vector<int>& tokens, torc
     const int n = static_cast<int>(tokens.size());
     k = checked_kv(k, n, "k");
     v = checked_kv(v, n, "v");
-    std::vector<Chunk*> fresh = tree_->reserve();
+    std::vector<Chunk*> fresh = reserve_and_note();
     refresh_kernel_context();
     {
         c10::DeviceGuard guard(t_options_.device());
@@ -158,7 +185,7 @@ std::vector<Chunk*> Attention::append_token_rotary(const std::vector<int>& token
         }
         pos = positions->data_ptr<int64_t>();
     }
-    std::vector<Chunk*> fresh = tree_->reserve();
+    std::vector<Chunk*> fresh = reserve_and_note();
     refresh_kernel_context();
     {
         c10::DeviceGuard guard(t_options_.device());

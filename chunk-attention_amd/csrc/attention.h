@@ -79,6 +79,11 @@ class Attention {
     std::unique_ptr<PrefixTree> tree_;
     ca_ctx* ctx_ = nullptr;
     uint64_t tables_version_ = 0;  // tree version the device tables were built from
+    // reserve() on a tree the tables were current for: the chunks it added, so that the next
+    // refresh patches the tables (ca_ctx_roll_tails) instead of rebuilding them from a tree walk
+    std::vector<Chunk*> reserve_and_note();
+    std::vector<int32_t> rolled_seqs_, rolled_slots_;
+    uint64_t rolled_version_ = 0;  // tree version right after that reserve(); 0 = nothing noted
 };
 
 // In-place rotary embedding of fp16 query/key rows: the operator the reference exports as

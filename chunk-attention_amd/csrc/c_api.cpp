@@ -76,18 +76,28 @@ struct ca_ctx {
     int delta_tokens = 0;
     int partition = 0;  // partition the current plan was built for
 
-    std::vector<ca::ChunkRow> rows;  // rows of the last refresh (to rebuild for another partition)
+    // rows of the last refresh (to rebuild for another partition, and for the reference-form
+    // tables).  Tail roll-overs patched into the plan since then are only logged: rows() replays
+    // the log when somebody asks for the rows.
+    mutable std::vector<ca::ChunkRow> rows;
+    struct Roll {
+        int delta_tokens;
+        std::vector<int32_t> seqs, slots;
+    };
+    mutable std::vector<Roll> pending_rolls;
     int n_seqs = 0;
     mutable ca::RefTables ref;  // reference-form tables of `rows`: use ref_tables(), never directly
     mutable bool ref_valid = false;
     ca::Plan plan;
 
-    // device tables: one blob, uploaded from one of two pinned staging buffers
+    // device tables: one blob, uploaded from a ring of pinned staging buffers (the host may run
+    // kStaging refreshes ahead of the device before it has to wait for a buffer)
+    static constexpr int kStaging = 4;
     char* dev_blob = nullptr;
     size_t dev_blob_cap = 0;
-    char* host_blob[2] = { nullptr, nullptr };
-    size_t host_blob_cap[2] = { 0, 0 };
-    hipEvent_t host_blob_free[2] = { nullptr, nullptr };
+    char* host_blob[kStaging] = {};
+    size_t host_blob_cap[kStaging] = {};
+    hipEvent_t host_blob_free[kStaging] = {};
     int next_host = 0;
     // offsets into dev_blob
     size_t off_shared = 0, off_stream = 0, off_slots = 0, off_seq_len = 0, off_part_ptr = 0,
@@ -104,6 +114,7 @@ struct ca_ctx {
     // hipFree waits for the whole device, so they are kept until the context is destroyed
     // (capacities double: together they never hold more than the live buffer does).
     std::vector<void*> retired;
+    std::vector<void*> retired_host;  // pinned staging buffers that were outgrown
 
     // optional timing: events recorded on the caller's stream around the launches.
     // 1: the fused launch; 2: forward run as three timed launches (chunk-first, sequence-first, merge)
@@ -165,8 +176,33 @@ int launch_rc(int rc, const char* what) {
     return fail_hip(static_cast<hipError_t>(rc), what);
 }
 
-// Builds the plan for `partition` from c->rows and uploads it.
-int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
+// Brings c->rows up to date with the roll-overs patched into the plan since the last refresh:
+// every sequence's last chunk gains the appended tokens, rolled sequences get their new empty
+// chunk as a row right after the old last one (where a pre-order walk of the tree puts it).
+const std::vector<ca::ChunkRow>& current_rows(const ca_ctx* c) {
+    for (const ca_ctx::Roll& roll : c->pending_rolls) {
+        std::vector<int> tail_row(c->n_seqs, -1);
+        for (size_t i = 0; i < c->rows.size(); i++) {
+            if (c->rows[i].seq_end - c->rows[i].seq_begin == 1) tail_row[c->rows[i].seq_begin] = static_cast<int>(i);
+        }
+        std::vector<int32_t> new_slot(c->n_seqs, -1);
+        for (size_t k = 0; k < roll.seqs.size(); k++) new_slot[roll.seqs[k]] = roll.slots[k];
+        std::vector<ca::ChunkRow> next;
+        next.reserve(c->rows.size() + roll.seqs.size());
+        for (size_t i = 0; i < c->rows.size(); i++) {
+            ca::ChunkRow r = c->rows[i];
+            const bool is_tail = r.seq_end - r.seq_begin == 1 && tail_row[r.seq_begin] == static_cast<int>(i);
+            if (is_tail) r.n_tokens += roll.delta_tokens;
+            next.push_back(r);
+            if (is_tail && new_slot[r.seq_begin] >= 0) next.push_back({ new_slot[r.seq_begin], 0, r.seq_begin, r.seq_end });
+        }
+        c->rows.swap(next);
+    }
+    c->pending_rolls.clear();
+    return c->rows;
+}
+
+ca::PlanParams plan_params(const ca_ctx* c, int partition) {
     ca::PlanParams pp;
     pp.tpp_threshold = c->tpp_threshold;
     pp.partition = partition;
@@ -175,9 +211,13 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     pp.n_heads = c->H;
     pp.n_cus = c->n_cus;
     pp.allow_per_wave = c->schedule == 0;  // the single-launch schedule synchronises workgroups
-    ca::build_plan(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, pp, &c->plan);
-    ca::Plan& p = c->plan;
+    return pp;
+}
 
+// Copies c->plan into a pinned staging buffer and queues its upload on `st`; sizes the
+// partial-row buffer for it.
+int upload_plan(ca_ctx* c, hipStream_t st) {
+    ca::Plan& p = c->plan;
     size_t off = 0;
     auto place = [&](size_t bytes) {
         const size_t at = off;
@@ -191,19 +231,19 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     c->off_part_ptr = place(p.part_ptr.size() * 4);
     c->off_tail_slot = place(p.tail_slot.size() * 4);
     c->off_tail_fill = place(p.tail_fill.size() * 4);
-    const size_t total = std::max<size_t>(off, 64);
+    const size_t total = std::max<size_t>(off, 64);  // a multiple of 64
 
     if (int rc = ensure_dev(c, &c->dev_blob, &c->dev_blob_cap, total)) return rc;
     const int hb = c->next_host;
-    c->next_host ^= 1;
+    c->next_host = (c->next_host + 1) % ca_ctx::kStaging;
     // the staging buffer may still be the source of an earlier asynchronous upload
     CA_HIP(hipEventSynchronize(c->host_blob_free[hb]));
     if (total > c->host_blob_cap[hb]) {
-        if (c->host_blob[hb]) CA_HIP(hipHostFree(c->host_blob[hb]));
-        c->host_blob[hb] = nullptr;
-        c->host_blob_cap[hb] = 0;
-        const size_t want = align_up(total + total / 4, 4096);
-        CA_HIP(hipHostMalloc(reinterpret_cast<void**>(&c->host_blob[hb]), want, hipHostMallocDefault));
+        const size_t want = align_up(std::max(total + total / 4, 2 * c->host_blob_cap[hb]), 4096);
+        void* fresh = nullptr;
+        CA_HIP(hipHostMalloc(&fresh, want, hipHostMallocDefault));
+        if (c->host_blob[hb]) c->retired_host.push_back(c->host_blob[hb]);  // freed with the context
+        c->host_blob[hb] = static_cast<char*>(fresh);
         c->host_blob_cap[hb] = want;
     }
     char* hbuf = c->host_blob[hb];
@@ -217,11 +257,21 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
     put(c->off_part_ptr, p.part_ptr.data(), p.part_ptr.size() * 4);
     put(c->off_tail_slot, p.tail_slot.data(), p.tail_slot.size() * 4);
     put(c->off_tail_fill, p.tail_fill.data(), p.tail_fill.size() * 4);
-    CA_HIP(hipMemcpyAsync(c->dev_blob, hbuf, total, hipMemcpyHostToDevice, st));
+    // a copy kernel, not hipMemcpyAsync: the copy engine's hand-over stalls the stream for
+    // several microseconds in the middle of a decode step
+    if (int rc = launch_rc(ca::launch_upload(c->dev_blob, hbuf, total, st), "table upload")) return rc;
     CA_HIP(hipEventRecord(c->host_blob_free[hb], st));
 
     const size_t part_bytes = std::max<size_t>(size_t(p.n_part_rows) * c->H * ca::PART_STRIDE * 4, 256);
-    if (int rc = ensure_dev(c, reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes)) return rc;
+    return ensure_dev(c, reinterpret_cast<char**>(&c->part), &c->part_cap, part_bytes);
+}
+
+// Builds the plan for `partition` from the context's rows and uploads it.
+int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
+    const std::vector<ca::ChunkRow>& rows = current_rows(c);
+    const ca::PlanParams pp = plan_params(c, partition);
+    ca::build_plan(rows.data(), static_cast<int>(rows.size()), c->n_seqs, c->C, pp, &c->plan);
+    if (int rc = upload_plan(c, st)) return rc;
     // completion counters (single-launch schedule only; a change of schedule rebuilds the plan and
     // comes through here): they start at zero, and each forward leaves them at zero again
     if (c->schedule != 0) {
@@ -237,7 +287,8 @@ int build_and_upload(ca_ctx* c, int partition, hipStream_t st) {
 // Reference-form tables of the rows the context holds, built on first use after a refresh.
 const ca::RefTables& ref_tables(const ca_ctx* c) {
     if (!c->ref_valid) {
-        ca::build_ref_tables(c->rows.data(), static_cast<int>(c->rows.size()), c->n_seqs, c->C, c->tpp_threshold, &c->ref);
+        const std::vector<ca::ChunkRow>& rows = current_rows(c);
+        ca::build_ref_tables(rows.data(), static_cast<int>(rows.size()), c->n_seqs, c->C, c->tpp_threshold, &c->ref);
         c->ref_valid = true;
     }
     return c->ref;
@@ -341,7 +392,7 @@ int ca_ctx_create(ca_ctx** out, int n_heads, int d_head, int chunk_size, void* k
         hipDeviceProp_t prop;
         if (err == hipSuccess) err = hipGetDeviceProperties(&prop, c->device);
         if (err == hipSuccess) c->n_cus = prop.multiProcessorCount;
-        for (int i = 0; i < 2 && err == hipSuccess; i++) {
+        for (int i = 0; i < ca_ctx::kStaging && err == hipSuccess; i++) {
             err = hipEventCreateWithFlags(&c->host_blob_free[i], hipEventDisableTiming);
         }
         // address of this device's static scratch (for ca_attention_noalloc), once per device
@@ -361,7 +412,8 @@ void ca_ctx_destroy(ca_ctx* c) {
     if (c->part) (void)hipFree(c->part);
     if (c->counters) (void)hipFree(c->counters);
     for (void* p : c->retired) (void)hipFree(p);
-    for (int i = 0; i < 2; i++) {
+    for (void* p : c->retired_host) (void)hipHostFree(p);
+    for (int i = 0; i < ca_ctx::kStaging; i++) {
         if (c->host_blob_free[i]) {
             (void)hipEventSynchronize(c->host_blob_free[i]);
             (void)hipEventDestroy(c->host_blob_free[i]);
@@ -386,11 +438,39 @@ int ca_refresh_kernel_context(ca_ctx* c, const ca_chunk_row* rows, int n_rows, i
             }
         }
         c->valid = false;
+        c->pending_rolls.clear();
         c->rows.resize(n_rows);
         if (n_rows) std::memcpy(c->rows.data(), rows, sizeof(ca_chunk_row) * n_rows);
         c->n_seqs = n_seqs;
         c->ref_valid = false;  // reference-form tables are for inspection: built when asked for
         if (int rc = build_and_upload(c, 0, static_cast<hipStream_t>(stream))) return rc;
+        c->delta_tokens = 0;
+        c->valid = true;
+        return CA_OK;
+    });
+}
+
+int ca_ctx_roll_tails(ca_ctx* c, const int32_t* seq_idx, const int32_t* new_slots, int n, void* stream) {
+    if (!c || n < 0 || (n > 0 && (!seq_idx || !new_slots))) return fail(CA_ERR_INVALID, "bad argument");
+    if (!c->valid) return fail(CA_ERR_STATE, "kernel context is not valid: call ca_refresh_kernel_context first");
+    if (c->schedule != c->plan_schedule) return fail(CA_ERR_STATE, "the tables were built for another schedule");
+    for (int i = 0; i < n; i++) {
+        if (new_slots[i] < 0 || new_slots[i] >= c->max_chunks) return fail(CA_ERR_INVALID, "slot outside the pool");
+    }
+    return guarded([&]() -> int {
+        try {
+            ca::roll_tails(&c->plan, c->C, plan_params(c, c->partition), c->delta_tokens, seq_idx, new_slots, n);
+        } catch (const std::invalid_argument& e) {
+            return fail(CA_ERR_STATE, e.what());  // plan untouched: the caller refreshes in full instead
+        }
+        ca_ctx::Roll roll;
+        roll.delta_tokens = c->delta_tokens;
+        roll.seqs.assign(seq_idx, seq_idx + n);
+        roll.slots.assign(new_slots, new_slots + n);
+        c->pending_rolls.push_back(std::move(roll));
+        c->ref_valid = false;
+        c->valid = false;
+        if (int rc = upload_plan(c, static_cast<hipStream_t>(stream))) return rc;
         c->delta_tokens = 0;
         c->valid = true;
         return CA_OK;
@@ -799,12 +879,15 @@ int ca_ctx_read_partials_raw(ca_ctx* c, float* out, int64_t n_floats, void* stre
 struct ca_tables {
     ca::RefTables ref;
     ca::Plan plan;
+    ca::PlanParams params;
     int n_seqs = 0;
+    int chunk_size = 0;
 };
 
-int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,
-                    int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks,
-                    int stream_chunks, int n_heads, int n_cus) {
+namespace {
+int tables_build(ca_tables** out, const ca_tables* like, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                 int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks, int stream_chunks,
+                 int n_heads, int n_cus) {
     if (!out || n_rows < 0 || n_seqs < 0 || (n_rows > 0 && !rows) || chunk_size <= 0) {
         return fail(CA_ERR_INVALID, "bad argument");
     }
@@ -812,14 +895,20 @@ int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n
     return guarded([&]() -> int {
         auto t = new ca_tables();
         t->n_seqs = n_seqs;
+        t->chunk_size = chunk_size;
         const ca::ChunkRow* r = reinterpret_cast<const ca::ChunkRow*>(rows);
-        ca::PlanParams pp;
+        ca::PlanParams& pp = t->params;
         pp.tpp_threshold = tpp_threshold;
         pp.partition = partition;
         pp.shared_seg_chunks = shared_seg_chunks;
         pp.stream_chunks = stream_chunks;
         pp.n_heads = n_heads;
         pp.n_cus = n_cus;
+        ca::PlanHints keep;
+        if (like) {
+            keep = like->plan.hints;
+            pp.keep = &keep;
+        }
         try {
             ca::build_ref_tables(r, n_rows, n_seqs, chunk_size, tpp_threshold, &t->ref);
             ca::build_plan(r, n_rows, n_seqs, chunk_size, pp, &t->plan);
@@ -827,7 +916,32 @@ int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n
             delete t;
             throw;
         }
+        pp.keep = nullptr;  // pointed at a local
         *out = t;
+        return CA_OK;
+    });
+}
+}  // namespace
+
+int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,
+                    int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks,
+                    int stream_chunks, int n_heads, int n_cus) {
+    return tables_build(out, nullptr, rows, n_rows, n_seqs, chunk_size, tpp_threshold, partition,
+                        shared_seg_chunks, stream_chunks, n_heads, n_cus);
+}
+
+int ca_tables_build_like(ca_tables** out, const ca_tables* like, const ca_chunk_row* rows, int n_rows,
+                         int n_seqs) {
+    if (!like) return fail(CA_ERR_INVALID, "bad argument");
+    const ca::PlanParams& pp = like->params;
+    return tables_build(out, like, rows, n_rows, n_seqs, like->chunk_size, pp.tpp_threshold, pp.partition,
+                        pp.shared_seg_chunks, pp.stream_chunks, pp.n_heads, pp.n_cus);
+}
+
+int ca_tables_roll_tails(ca_tables* t, int delta_tokens, const int32_t* seq_idx, const int32_t* new_slots, int n) {
+    if (!t) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        ca::roll_tails(&t->plan, t->chunk_size, t->params, delta_tokens, seq_idx, new_slots, n);
         return CA_OK;
     });
 }
@@ -950,6 +1064,20 @@ int ca_tree_reserve(ca_tree* t, int* n_new) {
     return guarded([&]() -> int {
         const auto fresh = t->tree.reserve();
         if (n_new) *n_new = static_cast<int>(fresh.size());
+        return CA_OK;
+    });
+}
+
+int ca_tree_reserve_tails(ca_tree* t, int32_t* seq_idx, int32_t* new_slots, int cap, int* n_new) {
+    if (!t) return fail(CA_ERR_INVALID, "null tree");
+    return guarded([&]() -> int {
+        std::vector<int> seqs;
+        const auto fresh = t->tree.reserve(&seqs);
+        if (n_new) *n_new = static_cast<int>(fresh.size());
+        for (int i = 0; i < static_cast<int>(fresh.size()) && i < cap; i++) {
+            if (seq_idx) seq_idx[i] = seqs[i];
+            if (new_slots) new_slots[i] = fresh[i]->slot();
+        }
         return CA_OK;
     });
 }

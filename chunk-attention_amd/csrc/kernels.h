@@ -52,6 +52,10 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
                   hipStream_t st);
 int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st);
 int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st);
+// Copies `bytes` (a multiple of 16) from pinned host memory to device memory with a kernel on
+// `st`.  For the table upload: a copy-engine transfer in the middle of a decode step costs the
+// stream several microseconds of hand-over between queues, a small kernel does not.
+int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream_t st);
 int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32_t* tail_slot,
                   const int32_t* tail_fill, int n_seqs, hipStream_t st);
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,

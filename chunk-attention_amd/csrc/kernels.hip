@@ -1097,6 +1097,11 @@ __global__ __launch_bounds__(WG) void fill_kernel(int32_t* __restrict__ p, int n
     if (idx < n) p[idx] = value;
 }
 
+__global__ __launch_bounds__(WG) void upload_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, int n) {
+    const int idx = blockIdx.x * WG + threadIdx.x;
+    if (idx < n) dst[idx] = src[idx];
+}
+
 // ---------------------------------------------------------------------------------------
 // K/V row writes.  One thread moves one piece (16 bytes when d_head allows, else 2) of K and V.
 // ---------------------------------------------------------------------------------------
@@ -1256,6 +1261,16 @@ int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st) {
 int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st) {
     if (n <= 0) return 0;
     hipLaunchKernelGGL(fill_kernel, dim3((n + WG - 1) / WG), dim3(WG), 0, st, p, n, value);
+    CA_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream_t st) {
+    if (bytes == 0) return 0;
+    if (bytes % 16 != 0 || bytes / 16 > size_t(1) << 30) return -1;
+    const int n = static_cast<int>(bytes / 16);
+    hipLaunchKernelGGL(upload_kernel, dim3((n + WG - 1) / WG), dim3(WG), 0, st, static_cast<uint4*>(dst_dev),
+                       static_cast<const uint4*>(src_pinned), n);
     CA_LAUNCH_CHECK();
     return 0;
 }

@@ -174,12 +174,14 @@ void PrefixTree::clear() {
     while (!tails_.empty()) remove_seq(static_cast<int>(tails_.size()) - 1);
 }
 
-std::vector<Chunk*> PrefixTree::reserve() {
+std::vector<Chunk*> PrefixTree::reserve(std::vector<int>* seq_idx) {
     std::vector<Chunk*> fresh;
-    for (auto& tail : tails_) {
+    for (size_t i = 0; i < tails_.size(); i++) {
+        Chunk*& tail = tails_[i];
         if (tail->full()) {
             Chunk* child = alloc_.allocate();
             fresh.push_back(child);
+            if (seq_idx) seq_idx->push_back(static_cast<int>(i));
             tail = tail->add_child(child);
         }
     }

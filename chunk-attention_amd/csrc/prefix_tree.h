@@ -94,8 +94,9 @@ class PrefixTree {
     void remove_seq(int seq_idx);
     // every sequence, highest index first (reference attention.cpp:280-285 intends this)
     void clear();
-    // reference attention.cpp:116-131
-    std::vector<Chunk*> reserve();
+    // reference attention.cpp:116-131.  seq_idx (optional): the index of the sequence each
+    // returned chunk became the last chunk of
+    std::vector<Chunk*> reserve(std::vector<int>* seq_idx = nullptr);
     // host half of reference attention.cpp:80-114: one token id per sequence.  Call
     // reserve() first; the K/V rows are written by the append kernel.
     void append_token_ids(const std::vector<int>& tokens);

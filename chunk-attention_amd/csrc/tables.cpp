@@ -54,11 +54,97 @@ namespace {
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 }  // namespace
 
+namespace {
+
+// Second stage of build_plan, also run on its own by roll_tails: cuts every sequence's private
+// chunks (Plan::own) into stream items, numbers the partial rows and decides the launch form.
+// Uses only what the plan holds, so that a patched plan and a rebuilt one agree.
+void build_stream_items(Plan& p, int chunk_size, const PlanParams& params) {
+    const int n_seqs = p.n_seqs;
+    p.slots.resize(p.n_shared_slots);
+    p.stream_items.clear();
+    std::vector<int32_t> n_parts = p.shared_parts;
+    const int stream_chunks = p.hints.stream_chunks, taper_chunks = p.hints.taper_chunks;
+    int n_streaming = 0;  // sequences that stream anything
+    for (int s = 0; s < n_seqs; s++) n_streaming += p.own[s].empty() ? 0 : 1;
+    const int generation = std::max(1, 2 * params.n_cus / std::max(params.n_heads, 1));
+    const int n_tapered = std::min(n_streaming / 2, std::max(n_streaming / 4, generation));
+    int rank = 0;
+    for (int s = 0; s < n_seqs; s++) {
+        const auto& own = p.own[s];
+        if (own.empty()) continue;
+        const int item_chunks = (taper_chunks > 0 && rank >= n_streaming - n_tapered) ? taper_chunks : stream_chunks;
+        rank++;
+        const int total = static_cast<int>(own.size());
+        // the last chunk is the sequence's tail, usually far from full: it rides along with
+        // the item before it instead of opening a new one
+        const int n_items = std::max(1, ceil_div(total - 1, item_chunks));
+        for (int g = 0; g < n_items; g++) {
+            const int c0 = int(int64_t(total) * g / n_items);
+            const int c1 = int(int64_t(total) * (g + 1) / n_items);
+            WorkItem it{};
+            it.seq_begin = s;
+            it.n_rows = 1;
+            it.slot_first = static_cast<int>(p.slots.size());
+            it.n_chunks = c1 - c0;
+            it.pos0 = p.own_pos0[s] + c0;
+            it.len0 = p.seq_len[s];
+            for (int k = c0; k < c1; k++) {
+                if (k - c0 < kInlineSlots) it.inl[k - c0] = own[k];
+                p.slots.push_back(own[k]);
+            }
+            it.part_row = n_parts[s]++;
+            p.stream_items.push_back(it);
+        }
+    }
+
+    // Many short runs (a long shared prompt, a few private tokens each): a workgroup per run
+    // would spend most of its life starting up, and only some of its waves would have a tile.
+    // When every item is at most three 64-token tiles and there are enough of them to fill the
+    // device at one item per wave, each wave takes an item of its own.
+    {
+        int max_tiles = 0;
+        for (const WorkItem& it : p.stream_items) max_tiles = std::max(max_tiles, ceil_div(it.n_chunks * chunk_size, 64));
+        const int64_t tasks = int64_t(p.stream_items.size()) * std::max(params.n_heads, 1);
+        p.stream_per_wave = params.allow_per_wave && !p.stream_items.empty() && max_tiles <= 3 &&
+                            tasks >= int64_t(3) * 2 * params.n_cus;
+    }
+
+    // a sequence whose only partial comes from a stream item needs no merge: that item
+    // writes the final output itself and its partial row is dropped from the merge list
+    for (auto& it : p.stream_items) {
+        if (n_parts[it.seq_begin] == 1) {
+            it.part_row = -1;
+            n_parts[it.seq_begin] = 0;
+        }
+    }
+
+    p.part_ptr.assign(n_seqs + 1, 0);
+    p.max_parts_per_seq = 0;
+    for (int s = 0; s < n_seqs; s++) {
+        p.part_ptr[s + 1] = p.part_ptr[s] + n_parts[s];
+        p.max_parts_per_seq = std::max(p.max_parts_per_seq, n_parts[s]);
+    }
+    p.n_part_rows = p.part_ptr[n_seqs];
+
+    // what the kernels assume about every item
+    for (const auto* list : { &p.shared_items, &p.stream_items }) {
+        for (const WorkItem& it : *list) {
+            if (it.n_chunks < 1 || it.n_chunks > kMaxItemChunks) {
+                throw std::logic_error("tables: work item with an unsupported number of chunks");
+            }
+        }
+    }
+}
+
+}  // namespace
+
 void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 const PlanParams& params, Plan* out) {
     Plan& p = *out;
     p = Plan();
     p.n_seqs = n_seqs;
+    p.partition = params.partition;
     p.seq_len.assign(n_seqs, 0);
     p.tail_slot.assign(n_seqs, -1);
     p.tail_fill.assign(n_seqs, 0);
@@ -149,6 +235,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     };
     int base_tiles = std::max(static_cast<int>(0.3 * step_us), 4);
     while (base_tiles < 32 && shared_wgs_with(base_tiles) > int64_t(2) * params.n_cus) base_tiles++;
+    if (params.keep) base_tiles = params.keep->base_tiles;
+    p.hints.base_tiles = base_tiles;
     auto seg_chunks_for = [&](bool wide) {
         if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
         const int n_tiles = std::min(base_tiles, wide ? 64 : 32);  // 64-token tiles
@@ -239,24 +327,39 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         }
     }
 
-    // ---- per-sequence stream items -------------------------------------------------------
-    std::vector<std::vector<int>> own_rows(n_seqs);
+    // ---- per-sequence private chunk lists -------------------------------------------------
+    p.n_shared_slots = static_cast<int>(p.slots.size());
+    p.own.assign(n_seqs, {});
+    p.own_pos0.assign(n_seqs, 0);
+    p.shared_parts = n_parts;
     int64_t stream_chunk_total = 0;
-    for (int i = 0; i < n_rows; i++) {
-        if (is_shared(rows[i])) continue;
-        for (int s = rows[i].seq_begin; s < rows[i].seq_end; s++) {
-            own_rows[s].push_back(i);
-            stream_chunk_total++;
+    {
+        std::vector<int> last_pos(n_seqs, -1);
+        for (int i = 0; i < n_rows; i++) {
+            if (is_shared(rows[i])) continue;
+            for (int s = rows[i].seq_begin; s < rows[i].seq_end; s++) {
+                // the chunks a sequence streams are the tail end of its path: consecutive positions
+                if (p.own[s].empty()) {
+                    p.own_pos0[s] = pos[i];
+                } else if (pos[i] != last_pos[s] + 1) {
+                    throw std::logic_error("tables: private chunks of a sequence are not consecutive");
+                }
+                last_pos[s] = pos[i];
+                p.own[s].push_back(rows[i].slot);
+                p.stream_tokens += rows[i].n_tokens;
+                stream_chunk_total++;
+            }
         }
     }
+    // Stream item length.  Taper: the stream items of the last sequences are half as long -- of
+    // as many sequences as fill the device's workgroup slots once (one "generation": 2 * n_cus /
+    // n_heads), or of the last quarter if that is more, never of more than half.  Workgroups
+    // start in item order, so these are the ones that run while the launch drains; with items of
+    // one size the last generation is a partial one whose members start late and end together
+    // (measured at 512 private tokens per sequence: 32 sequences 50.6 -> 49.5 us per forward, 48:
+    // 71.2 -> 69.7, 64: 88.6 -> 87.3, 128: 169.7 -> 167.3; quarter-length items leave waves idle
+    // and lose).
     int stream_chunks = params.stream_chunks;
-    // Taper: the stream items of the last sequences are half as long -- of as many sequences as
-    // fill the device's workgroup slots once (one "generation": 2 * n_cus / n_heads), or of the
-    // last quarter if that is more, never of more than half.  Workgroups start in item order, so
-    // these are the ones that run while the launch drains; with items of one size the last
-    // generation is a partial one whose members start late and end together (measured at 512
-    // private tokens per sequence: 32 sequences 50.6 -> 49.5 us per forward, 48: 71.2 -> 69.7,
-    // 64: 88.6 -> 87.3, 128: 169.7 -> 167.3; quarter-length items leave waves idle and lose).
     int taper_chunks = 0;
     if (stream_chunks <= 0) {
         // four waves per workgroup each take whole chunks, so prefer multiples of four;
@@ -274,82 +377,54 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     }
     stream_chunks = std::min(stream_chunks, kMaxItemChunks - 1);  // an item may take one chunk more
     if (taper_chunks >= stream_chunks) taper_chunks = 0;          // (after the cap: nothing to taper)
-    int n_streaming = 0;  // sequences that stream anything
-    for (int s = 0; s < n_seqs; s++) n_streaming += own_rows[s].empty() ? 0 : 1;
-    const int generation = std::max(1, 2 * params.n_cus / std::max(params.n_heads, 1));
-    const int n_tapered = std::min(n_streaming / 2, std::max(n_streaming / 4, generation));
-    int rank = 0;
-    for (int s = 0; s < n_seqs; s++) {
-        const auto& own = own_rows[s];
-        if (own.empty()) continue;
-        const int item_chunks = (taper_chunks > 0 && rank >= n_streaming - n_tapered) ? taper_chunks : stream_chunks;
-        rank++;
-        // the chunks a sequence streams are the tail end of its path: consecutive positions
-        for (size_t k = 1; k < own.size(); k++) {
-            if (pos[own[k]] != pos[own[k - 1]] + 1) {
-                throw std::logic_error("tables: private chunks of a sequence are not consecutive");
-            }
+    if (params.keep) {
+        stream_chunks = params.keep->stream_chunks;
+        taper_chunks = params.keep->taper_chunks;
+    }
+    p.hints.stream_chunks = stream_chunks;
+    p.hints.taper_chunks = taper_chunks;
+
+    build_stream_items(p, chunk_size, params);
+}
+
+void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_tokens,
+                const int32_t* seqs, const int32_t* new_slots, int n) {
+    Plan& p = *plan;
+    if (p.partition == 1 || params.tpp_threshold < 1 || params.partition != p.partition) {
+        throw std::invalid_argument("tables: this plan attends last chunks chunk-first, it cannot be patched");
+    }
+    if (delta_tokens < 0 || n < 0 || (n > 0 && (!seqs || !new_slots))) {
+        throw std::invalid_argument("tables: bad argument");
+    }
+    // validate before touching anything: the plan must stay usable when this throws
+    std::vector<char> rolls(p.n_seqs, 0);
+    for (int i = 0; i < n; i++) {
+        const int s = seqs[i];
+        if (s < 0 || s >= p.n_seqs || rolls[s]) throw std::invalid_argument("tables: bad or repeated sequence index");
+        if (p.tail_fill[s] + delta_tokens != chunk_size) {
+            throw std::invalid_argument("tables: the last chunk of a rolled sequence is not full");
         }
-        const int total = static_cast<int>(own.size());
-        // the last chunk is the sequence's tail, usually far from full: it rides along with
-        // the item before it instead of opening a new one
-        const int n_items = std::max(1, ceil_div(total - 1, item_chunks));
-        for (int g = 0; g < n_items; g++) {
-            const int c0 = int(int64_t(total) * g / n_items);
-            const int c1 = int(int64_t(total) * (g + 1) / n_items);
-            WorkItem it{};
-            it.seq_begin = s;
-            it.n_rows = 1;
-            it.slot_first = static_cast<int>(p.slots.size());
-            it.n_chunks = c1 - c0;
-            it.pos0 = pos[own[c0]];
-            it.len0 = p.seq_len[s];
-            for (int k = c0; k < c1; k++) {
-                if (k - c0 < kInlineSlots) it.inl[k - c0] = rows[own[k]].slot;
-                p.slots.push_back(rows[own[k]].slot);
-                p.stream_tokens += rows[own[k]].n_tokens;
-            }
-            it.part_row = n_parts[s]++;
-            p.stream_items.push_back(it);
+        if (p.own[s].empty()) throw std::invalid_argument("tables: sequence without a private last chunk");
+        rolls[s] = 1;
+    }
+    for (int s = 0; s < p.n_seqs; s++) {
+        if (!rolls[s] && p.tail_fill[s] + delta_tokens > chunk_size) {
+            throw std::invalid_argument("tables: a last chunk would hold more than chunk_size tokens");
         }
     }
-
-    // Many short runs (a long shared prompt, a few private tokens each): a workgroup per run
-    // would spend most of its life starting up, and only some of its waves would have a tile.
-    // When every item is at most three 64-token tiles and there are enough of them to fill the
-    // device at one item per wave, each wave takes an item of its own.
-    {
-        int max_tiles = 0;
-        for (const WorkItem& it : p.stream_items) max_tiles = std::max(max_tiles, ceil_div(it.n_chunks * chunk_size, 64));
-        const int64_t tasks = int64_t(p.stream_items.size()) * std::max(params.n_heads, 1);
-        p.stream_per_wave = params.allow_per_wave && !p.stream_items.empty() && max_tiles <= 3 &&
-                            tasks >= int64_t(3) * 2 * params.n_cus;
+    for (WorkItem& it : p.shared_items) it.len0 += delta_tokens;
+    for (int s = 0; s < p.n_seqs; s++) {
+        p.seq_len[s] += delta_tokens;
+        p.tail_fill[s] += delta_tokens;
     }
-
-    // a sequence whose only partial comes from a stream item needs no merge: that item
-    // writes the final output itself and its partial row is dropped from the merge list
-    for (auto& it : p.stream_items) {
-        if (n_parts[it.seq_begin] == 1) {
-            it.part_row = -1;
-            n_parts[it.seq_begin] = 0;
-        }
+    p.stream_tokens += int64_t(delta_tokens) * p.n_seqs;
+    for (int i = 0; i < n; i++) {
+        const int s = seqs[i];
+        p.own[s].push_back(new_slots[i]);
+        p.tail_slot[s] = new_slots[i];
+        p.tail_fill[s] = 0;
     }
-
-    p.part_ptr.assign(n_seqs + 1, 0);
-    for (int s = 0; s < n_seqs; s++) {
-        p.part_ptr[s + 1] = p.part_ptr[s] + n_parts[s];
-        p.max_parts_per_seq = std::max(p.max_parts_per_seq, n_parts[s]);
-    }
-    p.n_part_rows = p.part_ptr[n_seqs];
-
-    // what the kernels assume about every item
-    for (const auto* list : { &p.shared_items, &p.stream_items }) {
-        for (const WorkItem& it : *list) {
-            if (it.n_chunks < 1 || it.n_chunks > kMaxItemChunks) {
-                throw std::logic_error("tables: work item with an unsupported number of chunks");
-            }
-        }
-    }
+    build_stream_items(p, chunk_size, params);
 }
 
 }  // namespace ca

@@ -60,7 +60,17 @@ struct WorkItem {
 };
 static_assert(sizeof(WorkItem) == 64, "WorkItem must stay 64 bytes");
 
+// Decisions build_plan derives from the size of the whole step.  A plan patched after tails
+// rolled over keeps them (ca::roll_tails), and a rebuild can be told to (PlanParams::keep), so
+// that both give the same tables.
+struct PlanHints {
+    int base_tiles = 0;     // length of a shared segment in 64-token tiles before per-run adjustments
+    int stream_chunks = 0;  // chunks per stream item
+    int taper_chunks = 0;   // chunks per stream item of the last sequences, 0: no taper
+};
+
 struct PlanParams {
+    const PlanHints* keep = nullptr;  // reuse these instead of deriving them from the step's size
     int tpp_threshold = 1;
     int partition = 0;        // 0: shared chunks chunk-first, rest streamed; 1: all chunk-first;
                               // 2: everything streamed per sequence
@@ -92,9 +102,29 @@ struct Plan {
     std::vector<int32_t> part_ptr;   // [n_seqs + 1]: sequence s owns partial rows part_ptr[s] .. part_ptr[s+1]
     std::vector<int32_t> tail_slot;  // per sequence: slot of its last chunk
     std::vector<int32_t> tail_fill;  // per sequence: tokens in that chunk when built
+
+    // host-side state from which the stream items are (re)generated
+    PlanHints hints;
+    int partition = 0;                          // partition the plan was built for
+    int n_shared_slots = 0;                     // slots[0 .. n_shared_slots) belong to shared items
+    std::vector<std::vector<int32_t>> own;      // per sequence: slots of the chunks it streams, path order
+    std::vector<int32_t> own_pos0;              // per sequence: path position of own[s][0]
+    std::vector<int32_t> shared_parts;          // per sequence: partial rows written by shared items
 };
 
 void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 const PlanParams& params, Plan* out);
+
+// The tables after `delta_tokens` tokens were appended to every sequence since the plan was
+// built and the sequences seqs[i], whose last chunk is thereby full, each got the fresh empty
+// chunk new_slots[i] as new last chunk (reference Attention::reserve, attention.cpp:116-131).
+// Gives exactly what build_plan gives for the rows of the tree in that state with
+// PlanParams::keep = the plan's own hints: every length advances by delta_tokens, the rolled
+// sequences' stream items are cut again, partial-row numbering follows; shared items keep their
+// segments.  Only for plans in which no last chunk is attended chunk-first (partition 0 or 2
+// with tpp_threshold >= 1).  Throws std::invalid_argument when that does not hold or an argument
+// does not fit the plan; the plan is unchanged then.
+void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_tokens,
+                const int32_t* seqs, const int32_t* new_slots, int n);
 
 }  // namespace ca

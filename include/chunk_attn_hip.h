@@ -67,6 +67,19 @@ void ca_ctx_destroy(ca_ctx* ctx);
 int ca_refresh_kernel_context(ca_ctx* ctx, const ca_chunk_row* rows, int n_rows, int n_seqs,
                               void* stream);
 
+/* The refresh for the common decode-step case, without a tree walk: since the tables were built,
+ * delta_tokens tokens were appended to every sequence and nothing else changed, except that the
+ * sequences seq_idx[i] (whose last chunk is full now) each got the fresh empty chunk new_slots[i]
+ * as their new last chunk (what reference Attention::reserve does, attention.cpp:116-131; the
+ * reference then rebuilds every table, kernel_cuda.cu:1331-1445).  Patches the lengths, the rolled
+ * sequences' work items and the partial-row numbering in place, uploads, and resets delta_tokens
+ * to 0: the tables equal those of a full refresh that keeps the same work-item sizes.  n may be 0
+ * (folds delta_tokens into the tables).  CA_ERR_STATE when the tables cannot be patched (not
+ * valid, every chunk attended chunk-first, a listed chunk not full): they are left as they were,
+ * call ca_refresh_kernel_context instead. */
+int ca_ctx_roll_tails(ca_ctx* ctx, const int32_t* seq_idx, const int32_t* new_slots, int n,
+                      void* stream);
+
 /* KernelContext::valid / delta_tokens (kernel_cuda.h:42-45). */
 int ca_ctx_valid(const ca_ctx* ctx);
 void ca_ctx_invalidate(ca_ctx* ctx);
@@ -248,6 +261,13 @@ typedef struct ca_work_item {
 int ca_tables_build(ca_tables** out, const ca_chunk_row* rows, int n_rows, int n_seqs,
                     int chunk_size, int tpp_threshold, int partition, int shared_seg_chunks,
                     int stream_chunks, int n_heads, int n_cus);
+/* the same for other rows, reusing the work-item sizes `like` was built with instead of deriving
+ * them from the new rows (what a patched table keeps), and `like`'s other parameters */
+int ca_tables_build_like(ca_tables** out, const ca_tables* like, const ca_chunk_row* rows,
+                         int n_rows, int n_seqs);
+/* host half of ca_ctx_roll_tails on a built table set (the reference-form tables are not patched) */
+int ca_tables_roll_tails(ca_tables* t, int delta_tokens, const int32_t* seq_idx,
+                         const int32_t* new_slots, int n);
 void ca_tables_destroy(ca_tables* t);
 /* sizes: fills the same struct ca_ctx_plan_info fills */
 int ca_tables_info(const ca_tables* t, ca_plan_info* info);
@@ -286,6 +306,9 @@ int ca_tree_remove_seq(ca_tree* tree, int seq_idx);
 int ca_tree_clear(ca_tree* tree);
 /* reference Attention::reserve (attention.cpp:116-131); *n_new = chunks added */
 int ca_tree_reserve(ca_tree* tree, int* n_new);
+/* ca_tree_reserve that also reports, for each chunk added (up to cap), the index of the sequence
+ * it became the last chunk of and its slot: the arguments of ca_ctx_roll_tails */
+int ca_tree_reserve_tails(ca_tree* tree, int32_t* seq_idx, int32_t* new_slots, int cap, int* n_new);
 /* host half of reference Attention::append_token (attention.cpp:80-114): reserve, then
  * record one token id per sequence.  Returns *n_new like ca_tree_reserve. */
 int ca_tree_append_token(ca_tree* tree, const int32_t* tokens, int n_tokens, int* n_new);

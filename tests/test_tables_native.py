@@ -271,3 +271,73 @@ def test_all_shared_wide_runs_get_one_workgroup_per_compute_unit():
     assert len(half) == 4 and set(half[:, 3].tolist()) == {16}
     long_private = plan_for(0.75)
     assert len(long_private) == 1 and long_private[0, 3] == 48 and long_private[0, 7] == 1
+
+
+def assert_plans_equal(a: dict, b: dict):
+    assert sorted(a) == sorted(b)
+    for key in a:
+        if isinstance(a[key], np.ndarray):
+            np.testing.assert_array_equal(a[key], b[key], err_msg=key)
+        else:
+            assert a[key] == b[key], key
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_rolled_tables_equal_rebuilt_tables(seed):
+    """Decode steps on a random tree: whenever last chunks fill up, the tables patched in place
+    (ca_tables_roll_tails, the host half of ca_ctx_roll_tails) equal the tables built from a walk
+    of the tree in its new state with the same work-item sizes."""
+    rng = random.Random(100 + seed)
+    c = rng.choice([2, 4, 64])
+    partition = rng.choice([0, 0, 2])
+    tpp = rng.choice([1, 1, 2])
+    tree = capi.Tree(c, 4096)
+    fams = [[rng.randint(0, 3) for _ in range(rng.randint(c, 6 * c))] for _ in range(3)]
+    n = rng.randint(2, 12)
+    for s in range(n):
+        f = rng.choice(fams)
+        tree.add_seq(f[:rng.randint(1, len(f))] + [100 + 1000 * s + j for j in range(rng.randint(0, 3 * c))])
+    kw = dict(n_heads=rng.choice([2, 32]), n_cus=rng.choice([4, 256]))
+    first = capi.HostTables(tree.get_chunks(), n, c, tpp, partition, rng.choice([0, 0, 2]), rng.choice([0, 0, 3]), **kw)
+    live = capi.HostTables(tree.get_chunks(), n, like=first)
+    assert_plans_equal(live.plan(), first.plan())
+    delta, rolls = 0, 0
+    for step in range(3 * c + 5):
+        seqs, slots = tree.reserve_tails()
+        if seqs or step % 7 == 3:            # also: fold the appended tokens in with nothing rolled
+            live.roll_tails(delta, seqs, slots)
+            delta = 0
+            rolls += len(seqs)
+            rebuilt = capi.HostTables(tree.get_chunks(), n, like=first)
+            assert_plans_equal(live.plan(), rebuilt.plan())
+            check_plan(tree.get_chunks(), n, c, live.plan(), tpp, partition)
+        tree.append_token([5000 + step * 64 + s for s in range(n)])
+        delta += 1
+    assert rolls >= n
+
+
+def test_roll_tails_rejects_what_it_cannot_patch():
+    c = 4
+    tree = capi.Tree(c, 64)
+    tree.add_seq([1, 2, 3, 4, 5, 6])
+    tree.add_seq([1, 2, 3, 4, 7])
+    rows = tree.get_chunks()
+    t = capi.HostTables(rows, 2, c)
+    before = t.plan()
+    with pytest.raises(capi.ChunkAttnError):      # the last chunk of sequence 0 holds 2 of 4 tokens
+        t.roll_tails(0, [0], [9])
+    with pytest.raises(capi.ChunkAttnError):      # three more tokens do not fit sequence 0's last chunk
+        t.roll_tails(3, [], [])
+    with pytest.raises(capi.ChunkAttnError):
+        t.roll_tails(2, [0, 0], [9, 10])
+    with pytest.raises(capi.ChunkAttnError):
+        t.roll_tails(2, [5], [9])
+    assert_plans_equal(t.plan(), before)
+    t.roll_tails(2, [0], [9])                     # sequence 0 full after two tokens: fine
+    assert t.plan()["tail_slot"].tolist()[0] == 9 and t.plan()["tail_fill"].tolist() == [0, 3]
+    every_chunk_first = capi.HostTables(rows, 2, c, 1, 1)
+    with pytest.raises(capi.ChunkAttnError):
+        every_chunk_first.roll_tails(2, [0], [9])
+    last_chunks_shared = capi.HostTables(rows, 2, c, 0, 0)   # tpp_threshold 0: every chunk is attended chunk-first
+    with pytest.raises(capi.ChunkAttnError):
+        last_chunks_shared.roll_tails(2, [0], [9])
