@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -277,11 +278,15 @@ struct StreamPathLds {
     float l[NW];
     int state;  // workgroup-uniform decision flags
 };
-constexpr int KPITCH = D + 8;   // halves per LDS row of a K tile (272 B: rows stay 16-byte aligned)
+// K tiles use the same 288-byte row pitch: a 16-byte-per-lane read is served for lanes 0-7 of two
+// neighbouring 16-lane groups at a time, and with rows 288 B apart those sixteen pieces (rows i,
+// 16-byte columns g and g+1) fall into sixteen different 16-byte bank groups.  (272 B, which only
+// separates the rows of one group, costs every such read a second pass: measured with the LDS
+// bank-conflict counter.)
 constexpr int WROWS = 4 * MROWS;  // sequences per wide item: 32 per wave
 struct WidePathLds {
-    half_t k[64 * KPITCH];
-    half_t v[64 * VPITCH];
+    half_t k[1][64 * VPITCH];
+    half_t v[1][64 * VPITCH];
     int last[WROWS];
 };
 union __attribute__((aligned(16))) DecodeLds {
@@ -799,7 +804,34 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
 // tiles: all 256 threads stage the K and V tile in LDS once (the next tile is already on its way
 // in registers), then each wave runs the same MFMA scheme as shared_path with K operands read
 // from LDS.  Every K/V byte is fetched once per 128 sequences and no cross-wave merge is needed.
+//
+// What keeps the vector unit's share of a tile small (it, not the matrix cores, bounds the tile):
+//   * tiles that are wholly inside the sequence (all but at most the last) take a path with no
+//     validity tests at all; the last, partial tile zeroes the missing rows while staging and
+//     starts the score accumulators at -inf for the missing tokens instead of selecting afterwards;
+//   * row maxima cross the four 16-lane groups with the lane-swap instructions, not through LDS;
+//   * the running maximum only moves (and the accumulators are only rescaled) when some row of
+//     the wave finds a larger score: a wave-uniform test, false for most tiles after the first few;
+//   * the row sums come from one more matrix op per token pair (an all-ones A operand), which
+//     also sums exactly the fp16 probabilities that P.V uses.
 // ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float max_over_groups(float v) {
+    // lanes l, l^16, l^32, l^48 hold values of the same sequence: maximum of the four, in all four.
+    // The swap instructions exchange whole 16-lane rows between two registers (16: the odd rows
+    // of the first with the even rows of the second; 32: the upper half of the first with the lower
+    // half of the second); with two copies of one value the two results hold each lane's own value
+    // and its partner's.  (The result elements are copied out before the bit casts: a bit cast
+    // applied to a vector element directly reads element 0 whatever the index.)
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned a0 = a[0], a1 = a[1];
+    const float m16 = fmaxf(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
+    const unsigned w = __builtin_bit_cast(unsigned, m16);
+    const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    const unsigned b0 = b[0], b1 = b[1];
+    return fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
+}
+
 template <int C, int MBW>
 __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                           int h, WidePathLds& sm) {
@@ -824,177 +856,215 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
     const bool active = row_base < it.n_rows;       // wave has sequences (uniform per wave)
 
     h8 qreg[MB][4];
+    int prow[MB];  // partial row of this lane's sequence (needed at the very end: asked for now)
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
         const int row = row_base + mb * 16 + i;
         const half_t* qp = A.q + (size_t(it.seq_begin + row) * H + h) * D + 8 * g;
+        prow[mb] = (row < it.n_rows) ? A.part_ptr[it.seq_begin + row] + it.part_row : -1;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
         }
     }
-    float m_run[MB], l_lane[MB];
-    f4 oacc[MB][8];
+    float m_run[MB];
+    f4 oacc[MB][8], lacc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
         m_run[mb] = NEG_INF;
-        l_lane[mb] = 0.f;
+        lacc[mb] = f4{ 0.f, 0.f, 0.f, 0.f };
 #pragma unroll
         for (int db = 0; db < 8; db++) oacc[mb][db] = f4{ 0.f, 0.f, 0.f, 0.f };
     }
 
-    // tile t = tokens 64t .. 64t+63 of the segment.  Thread tid stages pieces tid + 256r
-    // (r = 0..3) of the K and of the V tile: piece p = row p/16, dims 8*(p%16) .. +7.
+    // The segment's tokens exist as a prefix: `have` of them, in n_full whole 64-token tiles and
+    // one partial tile of `rem` tokens.
     const int total_tokens = it.n_chunks * C;
-    const int n_tiles = (total_tokens + 63) / 64;
+    int have = len - it.pos0 * C;
+    have = have < total_tokens ? have : total_tokens;
+    have = have > 0 ? have : 0;
+    const int n_full = have >> 6, rem = have & 63;
+    const int n_tiles = n_full + (rem ? 1 : 0);
+
+    // Thread tid stages pieces tid + 256r (r = 0..3) of the K and of the V tile: piece p = token
+    // row p/16 of the tile, dims 8*(p%16) .. +7.  Sixteen token rows never straddle a chunk.
+    const int srow = tid >> 4, spiece = tid & 15;
+    const int lds_w = srow * VPITCH + 8 * spiece;
     uint4 kst[4], vst[4];
     auto fetch_tile = [&](int t) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int p = tid + 256 * r;
-            const int tok = 64 * t + (p >> 4);  // token of the segment
-            // the 16 token rows the workgroup stages in step r lie in one chunk (chunk sizes are
-            // multiples of 16): the chunk index is uniform
-            const int ck = (64 * t + 16 * r) / C;
-            const int valid = len - (it.pos0 + ck) * C - (tok % C);  // > 0: token exists
-            if (tok < total_tokens && valid > 0) {
-                const size_t off = ((size_t(chunk_slot(slotv, ck)) * H + h) * size_t(C) + (tok % C)) * D + 8 * (p & 15);
-                kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
-                vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
+            int ck, crow;  // chunk of the item and token row inside it
+            if constexpr (C == 64) {
+                ck = t; crow = srow + 16 * r;
+            } else if constexpr (C == 128) {
+                ck = t >> 1; crow = 64 * (t & 1) + srow + 16 * r;
             } else {
-                kst[r] = make_uint4(0, 0, 0, 0);  // missing tokens: zero V, scores masked below
-                vst[r] = make_uint4(0, 0, 0, 0);
+                ck = 2 * t + (r >> 1); crow = srow + 16 * (r & 1);
             }
+            // a chunk index past the item's last chunk reads lane values that were preloaded as
+            // slot 0: valid memory, and only ever for tokens the partial-tile path zeroes
+            const size_t off = ((size_t(chunk_slot(slotv, ck & 63)) * H + h) * size_t(C) + crow) * D + 8 * spiece;
+            kst[r] = *reinterpret_cast<const uint4*>(kpool + off);
+            vst[r] = *reinterpret_cast<const uint4*>(vpool + off);
         }
     };
-    // number of existing tokens in tile t (tokens exist as a prefix of the segment)
-    auto tile_valid = [&](int t) {
-        int have = len - it.pos0 * C - 64 * t;
-        const int cap = total_tokens - 64 * t;
-        have = have < cap ? have : cap;
-        return have < 64 ? have : 64;
-    };
+    h8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ones[e] = half_t(1.f);
 
-    if (n_tiles > 0) fetch_tile(0);
-    for (int t = 0; t < n_tiles; t++) {
-        const int valid = tile_valid(t);
-        if (valid <= 0) break;  // uniform: nothing further exists
-        __syncthreads();        // everyone is done reading the previous tile
+    // MASKED: the tile holds only `valid` (< 64) tokens.  Rows past them hold stale data: zeroed
+    // on their way into LDS (V must not meet a NaN), their scores start at -inf.
+    // stage the tile held in kst/vst into buffer `buf`; valid < 64: rows past the tile's tokens
+    // are zeroed on their way in
+    auto stage_tile = [&](int buf, int valid) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int p = tid + 256 * r;
-            *reinterpret_cast<uint4*>(&sm.k[(p >> 4) * KPITCH + 8 * (p & 15)]) = kst[r];
-            *reinterpret_cast<uint4*>(&sm.v[(p >> 4) * VPITCH + 8 * (p & 15)]) = vst[r];
+            uint4 kk = kst[r], vv = vst[r];
+            if (srow + 16 * r >= valid) {
+                kk = make_uint4(0, 0, 0, 0);
+                vv = make_uint4(0, 0, 0, 0);
+            }
+            *reinterpret_cast<uint4*>(&sm.k[buf][lds_w + 16 * r * VPITCH]) = kk;
+            *reinterpret_cast<uint4*>(&sm.v[buf][lds_w + 16 * r * VPITCH]) = vv;
+        }
+    };
+    auto stage_full_tile = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            *reinterpret_cast<uint4*>(&sm.k[buf][lds_w + 16 * r * VPITCH]) = kst[r];
+            *reinterpret_cast<uint4*>(&sm.v[buf][lds_w + 16 * r * VPITCH]) = vst[r];
+        }
+    };
+
+    // One tile: staged from kst/vst between two barriers, then the next tile is requested and this
+    // one is attended.  (Staging the next tile into a second buffer while this one is read, one
+    // barrier per tile, measured slower: 99.8 against 76.1 us for a 64-tile segment.)
+    // MASKED: the tile holds only `valid` (< 64) tokens: their scores start at -inf (the staging
+    // zeroed the rows, so stale NaNs never meet V).
+    auto tile_body = [&](int t, auto masked_tag, int valid) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const half_t* __restrict__ kt = sm.k[0];
+        const half_t* __restrict__ vt = sm.v[0];
+        __syncthreads();
+        if (MASKED) {
+            stage_tile(0, valid);
+        } else {
+            stage_full_tile(0);
         }
         __syncthreads();
         if (t + 1 < n_tiles) fetch_tile(t + 1);
-        if (!active) continue;
-
-        // scores of the 64 tokens for this wave's rows
-        f4 sc[MB][4];
+        if (active) {
+            // scores of the 64 tokens for this wave's rows; lane (g, i) gets tokens 16tb + 4g .. +3
+            // of sequence row i
+            f4 sc[MB][4];
 #pragma unroll
-        for (int tb = 0; tb < 4; tb++) {
-            h8 kop[4];
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                kop[ks] = *reinterpret_cast<const h8*>(&sm.k[(16 * tb + i) * KPITCH + 32 * ks + 8 * g]);
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                // rows past the item's last sequence carry zero queries: computed, never stored
-                // (no branch in this loop, so that LDS reads and matrix ops can be pipelined)
-                f4 acc = f4{ 0.f, 0.f, 0.f, 0.f };
+            for (int tb = 0; tb < 4; tb++) {
+                h8 kop[4];
 #pragma unroll
                 for (int ks = 0; ks < 4; ks++) {
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[ks], qreg[mb][ks], acc, 0, 0, 0);
+                    kop[ks] = *reinterpret_cast<const h8*>(&kt[(16 * tb + i) * VPITCH + 32 * ks + 8 * g]);
                 }
-                sc[mb][tb] = acc;
-            }
-        }
-        // online softmax on the raw scores: the row maximum is taken before scaling (the scale
-        // is positive) and the scale rides in the exponent's multiply-add.  Tokens past the end
-        // of the sequence are masked with selects, never with a branch: no branch may sit
-        // between a matrix op and the first use of its result (the wait states the compiler
-        // inserts for that hazard do not reach across a taken branch).
+                f4 init = f4{ 0.f, 0.f, 0.f, 0.f };
+                if constexpr (MASKED) {
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-#pragma unroll
-            for (int tb = 0; tb < 4; tb++) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (16 * tb + 4 * g + r >= valid) sc[mb][tb][r] = NEG_INF;
+                    for (int r = 0; r < 4; r++) init[r] = (16 * tb + 4 * g + r >= valid) ? NEG_INF : 0.f;
                 }
-            }
-        }
-        h4 pb[MB][4];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            float mx = NEG_INF;
-#pragma unroll
-            for (int tb = 0; tb < 4; tb++) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) mx = fmaxf(mx, sc[mb][tb][r]);
-            }
-            mx = fmaxf(mx, shfl_xor(mx, 16));
-            mx = fmaxf(mx, shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run[mb], mx * scale_log2);  // valid >= 1: mx is finite
-            const float alpha = fast_exp2(m_run[mb] - m_new);
-            m_run[mb] = m_new;
-            float psum = 0.f;
-#pragma unroll
-            for (int tb = 0; tb < 4; tb++) {
-                float p[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    p[r] = fast_exp2(__builtin_fmaf(sc[mb][tb][r], scale_log2, -m_new));
-                    psum += p[r];
-                }
-                pb[mb][tb] = h4{ half_t(p[0]), half_t(p[1]), half_t(p[2]), half_t(p[3]) };
-            }
-            l_lane[mb] = l_lane[mb] * alpha + psum;
-#pragma unroll
-            for (int db = 0; db < 8; db++) oacc[mb][db] *= alpha;
-        }
-        // O^T += V^T . P^T with k = 32 tokens per instruction: k-slot (g, e) stands for token
-        // 4g + e of 16-token block 2*tp (e < 4) or 2*tp + 1 (e >= 4) in both operands, which is
-        // where the S^T result layout already holds the probabilities
-#pragma unroll
-        for (int tp = 0; tp < 2; tp++) {
-            h8 pp[MB];
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                const h4 lo = pb[mb][2 * tp], hi = pb[mb][2 * tp + 1];
-                pp[mb] = h8{ lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-            }
-            // all eight V^T operands of this token pair are requested before the first matrix
-            // op waits for one: the reads' latencies overlap instead of adding up
-            h8 a[8];
-#pragma unroll
-            for (int db = 0; db < 8; db++) {
-                const half_t* p0 = &sm.v[(32 * tp + 4 * g + (i >> 2)) * VPITCH + 16 * db + 4 * (i & 3)];
-                const h4 lo = lds_read_tr(p0), hi = lds_read_tr(p0 + 16 * VPITCH);
-                a[db] = h8{ lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int db = 0; db < 8; db++) {
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++) {
-                    oacc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[mb], oacc[mb][db], 0, 0, 0);
+                    // rows past the item's last sequence carry zero queries: computed, never stored
+                    f4 acc = init;
+#pragma unroll
+                    for (int ks = 0; ks < 4; ks++) {
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[ks], qreg[mb][ks], acc, 0, 0, 0);
+                    }
+                    sc[mb][tb] = acc;
+                }
+            }
+            // Online softmax on the raw scores: the row maximum is taken before scaling (the scale is
+            // positive) and the scale rides in the exponent's multiply-add.  No branch sits between a
+            // matrix op and the first use of its result: the one branch below follows the maxima.
+            float m_new[MB];
+            bool grew = false;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                float mx = fmaxf(fmaxf(sc[mb][0][0], sc[mb][0][1]), fmaxf(sc[mb][0][2], sc[mb][0][3]));
+#pragma unroll
+                for (int tb = 1; tb < 4; tb++) {
+                    mx = fmaxf(mx, fmaxf(fmaxf(sc[mb][tb][0], sc[mb][tb][1]), fmaxf(sc[mb][tb][2], sc[mb][tb][3])));
+                }
+                mx = max_over_groups(mx);  // valid >= 1: finite
+                m_new[mb] = fmaxf(m_run[mb], mx * scale_log2);
+                grew |= m_new[mb] > m_run[mb];
+            }
+            if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+                // some row of the wave found a larger score: move the maxima, rescale what was summed
+                // relative to the old ones (rows that did not move get a factor of exactly 1)
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    const float alpha = fast_exp2(m_run[mb] - m_new[mb]);
+                    m_run[mb] = m_new[mb];
+                    lacc[mb] *= alpha;
+#pragma unroll
+                    for (int db = 0; db < 8; db++) oacc[mb][db] *= alpha;
+                }
+            }
+            // Per pair of 16-token blocks: probabilities, packed as the B operand of the 32-token-
+            // deep P.V (k-slot (g, e) stands for token 4g + e of block 2*tp (e < 4) or 2*tp + 1
+            // (e >= 4), which is where the S^T result layout already holds them), then the matrix ops
+            // of that pair; the second pair's exponentials do not depend on the first pair's
+            // matrix ops and stand between them in program order, so that they can overlap.
+            h8 pp[MB][2];
+            auto probabilities = [&](int tp) {
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    const float nm = -m_run[mb];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        pp[mb][tp][e] = half_t(fast_exp2(__builtin_fmaf(sc[mb][2 * tp + (e >> 2)][e & 3], scale_log2, nm)));
+                    }
+                }
+            };
+            probabilities(0);
+#pragma unroll
+            for (int tp = 0; tp < 2; tp++) {
+                // all eight V^T operands of this token pair are requested before the first matrix
+                // op waits for one: the reads' latencies overlap instead of adding up
+                h8 a[8];
+#pragma unroll
+                for (int db = 0; db < 8; db++) {
+                    const half_t* p0 = &vt[(32 * tp + 4 * g + (i >> 2)) * VPITCH + 16 * db + 4 * (i & 3)];
+                    const h4 lo = lds_read_tr(p0), hi = lds_read_tr(p0 + 16 * VPITCH);
+                    a[db] = h8{ lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+                }
+                if (tp == 0) probabilities(1);
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    // row sums: an all-ones A operand adds up the probabilities of every sequence
+                    lacc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pp[mb][tp], lacc[mb], 0, 0, 0);
+                }
+#pragma unroll
+                for (int db = 0; db < 8; db++) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++) {
+                        oacc[mb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[db], pp[mb][tp], oacc[mb][db], 0, 0, 0);
+                    }
                 }
             }
         }
-    }
+    };
+
+    if (n_tiles > 0) fetch_tile(0);
+    for (int t = 0; t < n_full; t++) tile_body(t, std::false_type{}, 64);
+    if (rem) tile_body(n_full, std::true_type{}, rem);
 
     // ---- each wave writes the partial rows of its own sequences ----------------------------
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
-        l_lane[mb] += shfl_xor(l_lane[mb], 16);
-        l_lane[mb] += shfl_xor(l_lane[mb], 32);
-        const int row = row_base + mb * 16 + i;
-        if (row < it.n_rows) {
-            float* dst = A.part + (size_t(A.part_ptr[it.seq_begin + row] + it.part_row) * H + h) * PART_STRIDE;
-            if (g == 0) part_store2(dst, m_run[mb], l_lane[mb], coh);
+        if (prow[mb] >= 0) {
+            float* dst = A.part + (size_t(prow[mb]) * H + h) * PART_STRIDE;
+            // every lane of a sequence holds the same row sum (the matrix op summed over all tokens)
+            if (g == 0) part_store2(dst, m_run[mb], lacc[mb][0], coh);
 #pragma unroll
             for (int db = 0; db < 8; db++) {
                 part_store2(dst + 4 + 16 * db + 4 * g, oacc[mb][db][0], oacc[mb][db][1], coh);
