@@ -127,11 +127,13 @@ struct ca_ctx {
 
 namespace {
 
-// Makes *p hold at least `need` bytes.  Growth at least doubles the capacity and retires the old
-// buffer instead of freeing it: nothing on the decode step's path waits for the device.
+// Makes *p hold at least `need` bytes.  A new buffer is twice what is asked for (tables and
+// partial rows grow step by step while sequences grow, and an allocation in the middle of a
+// decode loop costs the host hundreds of microseconds); the old one is retired instead of freed:
+// nothing on the decode step's path waits for the device.
 int ensure_dev(ca_ctx* c, char** p, size_t* cap, size_t need) {
     if (need <= *cap) return CA_OK;
-    const size_t want = align_up(std::max(need + need / 4, 2 * *cap), 4096);
+    const size_t want = align_up(std::max(2 * need, 2 * *cap), 4096);
     void* fresh = nullptr;
     CA_HIP(hipMalloc(&fresh, want));
     if (*p) c->retired.push_back(*p);
@@ -236,16 +238,22 @@ int upload_plan(ca_ctx* c, hipStream_t st) {
     if (int rc = ensure_dev(c, &c->dev_blob, &c->dev_blob_cap, total)) return rc;
     const int hb = c->next_host;
     c->next_host = (c->next_host + 1) % ca_ctx::kStaging;
+    if (total > c->host_blob_cap[hb]) {
+        // the whole ring grows at once, with headroom: pinned allocations cost the host a hundred
+        // microseconds each and must not recur on the following decode steps
+        const size_t want = align_up(std::max(2 * total, 2 * c->host_blob_cap[hb]), 4096);
+        for (int b = 0; b < ca_ctx::kStaging; b++) {
+            if (c->host_blob_cap[b] >= want) continue;
+            void* fresh = nullptr;
+            CA_HIP(hipHostMalloc(&fresh, want, hipHostMallocDefault));
+            // the old buffer may still be the source of a queued upload: freed with the context
+            if (c->host_blob[b]) c->retired_host.push_back(c->host_blob[b]);
+            c->host_blob[b] = static_cast<char*>(fresh);
+            c->host_blob_cap[b] = want;
+        }
+    }
     // the staging buffer may still be the source of an earlier asynchronous upload
     CA_HIP(hipEventSynchronize(c->host_blob_free[hb]));
-    if (total > c->host_blob_cap[hb]) {
-        const size_t want = align_up(std::max(total + total / 4, 2 * c->host_blob_cap[hb]), 4096);
-        void* fresh = nullptr;
-        CA_HIP(hipHostMalloc(&fresh, want, hipHostMallocDefault));
-        if (c->host_blob[hb]) c->retired_host.push_back(c->host_blob[hb]);  // freed with the context
-        c->host_blob[hb] = static_cast<char*>(fresh);
-        c->host_blob_cap[hb] = want;
-    }
     char* hbuf = c->host_blob[hb];
     auto put = [&](size_t at, const void* src, size_t bytes) {
         if (bytes) std::memcpy(hbuf + at, src, bytes);
