@@ -152,7 +152,7 @@ def pybind_forward_us(w, q, steps, warmup, torch, seed):
     (us per forward, us per forward of the C-ABI call on the same cache with a preallocated output)."""
     import numpy as np
     import chunk_attn
-    attn = pybind_cache(w, torch, seed, extra_chunks_per_seq=6)
+    attn = pybind_cache(w, torch, seed, extra_chunks_per_seq=10)
     for _ in range(warmup):
         out = attn.forward(q)
     torch.cuda.synchronize()
@@ -176,9 +176,9 @@ def pybind_forward_us(w, q, steps, warmup, torch, seed):
         rebuild_us += (time.perf_counter() - t0) * 1e6 / 15
     torch.cuda.synchronize()
     kz = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
-    reserve_us, roll_us, n_rolled, rolls = 0.0, 0.0, 0, 0
+    reserve_t, roll_t, n_rolled, rolls = [], [], 0, 0
     c = w.chunk_size
-    for t in range(5 * c):
+    for t in range(8 * c):
         attn.append_token([1_900_000_000 - t * 4096 - s for s in range(w.n_seqs)], kz, kz)
         if any(x.n_tokens == c for x in attn.tails):     # full last chunks: the next reserve rolls them
             # (no device sync in front: the first launch after one costs the host 10 us more)
@@ -188,19 +188,21 @@ def pybind_forward_us(w, q, steps, warmup, torch, seed):
             attn.refresh_kernel_context()                # the tables: patched in place, upload queued
             t2 = time.perf_counter()
             if rolls or t >= c:                          # the first patch is not timed
-                reserve_us += (t1 - t0) * 1e6
-                roll_us += (t2 - t1) * 1e6
+                reserve_t.append((t1 - t0) * 1e6)
+                roll_t.append((t2 - t1) * 1e6)
                 n_rolled += len(fresh)
             rolls += 1
     torch.cuda.synchronize()
     timed = max(rolls - 1, 1)
-    tables = {"tree_changed_us": round(rebuild_us, 1), "tails_rolled_us": round(roll_us / timed, 1),
-              "reserve_call_us": round(reserve_us / timed, 1),
+    tables = {"tree_changed_us": round(rebuild_us, 1), "tails_rolled_us": round(float(np.median(roll_t)), 1),
+              "tails_rolled_max_us": round(max(roll_t), 1),
+              "reserve_call_us": round(float(np.median(reserve_t)), 1),
               "tails_rolled_per_patch": n_rolled // timed, "patches_timed": rolls - 1,
               "note": "host time per call through chunk_attn.Attention; tree_changed = refresh_kernel_context(True): tree "
                       "walk + tables + upload; tails_rolled = refresh_kernel_context() after reserve() gave full last "
                       "chunks a successor: tables patched in place + upload (reserve_call_us is that reserve(), which "
-                      "also builds one Python object per new chunk)"}
+                      "also builds one Python object per new chunk); medians over the patches timed, max = the "
+                      "patch that outgrew a device buffer, if one did (buffers double)"}
     return us, out, tables
 
 
