@@ -122,27 +122,31 @@ def cold_forward_us(attn, q, out, torch, reps=20, hints=(("default_policy", 0), 
     return res
 
 
-def plain_read_gbps(n_bytes, torch, reps=20):
-    """What a read with no structure reaches on this GPU: torch's sum over an int64 buffer of
+def plain_read_gbps(ctx, n_bytes, torch, reps=20):
+    """What a read with no structure reaches on this GPU: the library's read probe (one
+    workgroup per compute unit, non-temporal 16-byte loads, nothing kept) over a buffer of
     n_bytes, repeated back to back (warm) and after a read of 1 GiB of other memory (cold), HIP
-    events around the sum.  A yardstick beside the published peak, not a replacement for it."""
-    buf = torch.ones(max(n_bytes // 8, 1), dtype=torch.int64, device="cuda:0")
+    events around the launch; and over 2 GiB, where no cache helps and the launch's start and end
+    no longer weigh.  A yardstick beside the published peak, not a replacement for it."""
+    stream = torch.cuda.current_stream().cuda_stream
     flush = torch.zeros(1 << 27, dtype=torch.int64, device="cuda:0")
     res = {}
-    for name in ("warm", "cold"):
+    for name, size, cold in (("warm", n_bytes, False), ("cold", n_bytes, True), ("2GiB", 2 << 30, False)):
+        buf = torch.ones(max(size // 8, 2), dtype=torch.int64, device="cuda:0")
         total = 0.0
         for i in range(reps + 2):
-            if name == "cold":
+            if cold:
                 flush.sum()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            buf.sum()
+            ctx.read_probe(buf.data_ptr(), buf.numel() * 8, stream)
             e1.record()
             e1.synchronize()
             if i >= 2:
                 total += e0.elapsed_time(e1)
         res[name] = round(buf.numel() * 8 / (total * 1e-3 / reps) / 1e9, 1)
-    del buf, flush
+        del buf
+    del flush
     return res
 
 
@@ -552,9 +556,10 @@ def main() -> int:
         result["roofline"]["fits_last_level_cache"] = bool(stream_bytes + shared_bytes <= (256 << 20))
         result["roofline"]["cold_note"] = ("decode launch after 1 GiB of other memory was read, HIP events recorded inside "
                                            "the library around that launch (they add about 2 us: the fraction is a lower bound)")
-        result["roofline"]["plain_read_GBps"] = plain_read_gbps(decode_bytes, torch)
-        result["roofline"]["plain_read_note"] = ("torch.sum over an int64 buffer of bytes_per_launch bytes under the same two "
-                                                 "protocols (repeated; after the 1 GiB read), HIP events around the call")
+        result["roofline"]["plain_read_GBps"] = plain_read_gbps(attn.ctx, decode_bytes, torch)
+        result["roofline"]["plain_read_note"] = ("a kernel that only reads (non-temporal 16-byte loads, one workgroup per compute "
+                                                 "unit) over bytes_per_launch bytes under the same two protocols (repeated; after "
+                                                 "the 1 GiB read) and over 2 GiB, HIP events around the launch")
     if not args.no_pybind:
         pyb_us, pyb_out, pyb_tables = pybind_forward_us(w, q, args.steps, args.warmup, torch, args.seed)
         torch.cuda.synchronize()

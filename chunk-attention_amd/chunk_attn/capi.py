@@ -82,7 +82,9 @@ SIGNATURES = {
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
     "ca_ctx_set_schedule": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_set_stream_hint": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_set_markers": (ctypes.c_int, [ctypes.c_int]),
     "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_ctx_read_probe": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "ca_ctx_read_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_int64), ctypes.c_int]),
@@ -153,6 +155,11 @@ class ChunkAttnError(RuntimeError):
 def _check(rc: int) -> None:
     if rc != 0:
         raise ChunkAttnError(rc, load().ca_last_error().decode())
+
+
+def set_markers(enable: bool) -> None:
+    """Named ranges (roctx) around refreshes, patches, attention calls and appends; off by default."""
+    _check(load().ca_set_markers(1 if enable else 0))
 
 
 def _i32(values: Sequence[int]):
@@ -544,6 +551,10 @@ class KernelContext:
         """0 off, 1 time the fused launch, 2 run and time the three phases separately, 3 / 4 issue only
         the decode launch / only its sequence-first workgroups (for timing a train of them)."""
         _check(self._lib.ca_ctx_set_timing(self._h, int(mode)))
+
+    def read_probe(self, dev_ptr: int, n_bytes: int, stream: int = 0) -> None:
+        """Measurement aid: one launch that reads n_bytes of device memory and keeps nothing."""
+        _check(self._lib.ca_ctx_read_probe(self._h, dev_ptr, n_bytes, stream))
 
     def read_timing(self, reset: bool = True) -> dict:
         """Accumulated per-phase milliseconds of the timed ca_attention calls."""

@@ -31,27 +31,29 @@ class ModelHost:
         self.peak_batch_size = 0
         self.iterations = 0
         self.stopped = True
-        self.cycle_time = 1.0
-        # double queue size to avoid blocking
+        self.cycle_time = 1.0               # seconds an idle worker waits for a request per round
+        # room for a whole batch beyond the one being admitted: producers rarely wait on put()
         self.batch_queue: "queue.Queue[Sequence]" = queue.Queue(maxsize=2 * max_batch_size)
         self.thread: Optional[threading.Thread] = None
 
     def predict_async(self, prompt_tokens: List[int], max_tokens: int) -> Sequence:
+        """Queues a request; the returned Sequence delivers tokens (or the error) when done."""
+        request = Sequence(prompt_tokens=prompt_tokens, max_tokens=max_tokens)
         if self.stopped:
-            raise RuntimeError("model host is stopped, can't predict anymore")
-        seq = Sequence(prompt_tokens=prompt_tokens, max_tokens=max_tokens)
-        self.batch_queue.put(seq)
-        return seq
+            raise RuntimeError("model host is stopped: start() it before asking for predictions")
+        self.batch_queue.put(request)
+        return request
 
     def predict(self, prompt_tokens: List[int], max_tokens: int) -> List[int]:
         return self.predict_async(prompt_tokens, max_tokens).get_result()
 
     def start(self) -> None:
-        if not self.stopped:
+        if self.thread is not None or not self.stopped:
             raise RuntimeError("model host is already started")
+        worker = threading.Thread(target=self.run_iterations, name="chunk-attn-model-host", daemon=True)
         self.stopped = False
-        self.thread = threading.Thread(target=self.run_iterations, daemon=True)
-        self.thread.start()
+        self.thread = worker
+        worker.start()
 
     def stop(self) -> None:
         self.stopped = True
@@ -60,21 +62,22 @@ class ModelHost:
             self.thread = None
 
     def get_new_requests(self) -> List[Sequence]:
-        new_seqs: List[Sequence] = []
-        # nothing running: block until at least one request arrives (or the cycle ends)
-        if len(self.running_seqs) == 0:
+        """Requests to admit this iteration: as many as fit beside the running sequences.  An idle
+        host waits up to cycle_time for the first one instead of spinning."""
+        room = self.max_batch_size - len(self.running_seqs)
+        admitted: List[Sequence] = []
+        wait = self.cycle_time if not self.running_seqs else None
+        while len(admitted) < room:
             try:
-                new_seqs.append(self.batch_queue.get(block=True, timeout=self.cycle_time))
-            except queue.Empty:
-                pass
-        while len(new_seqs) + len(self.running_seqs) < self.max_batch_size and not self.batch_queue.empty():
-            try:
-                new_seqs.append(self.batch_queue.get(block=False))
+                if wait is not None and not admitted:
+                    admitted.append(self.batch_queue.get(timeout=wait))
+                else:
+                    admitted.append(self.batch_queue.get_nowait())
             except queue.Empty:
                 break
         if self.prefix_aware:
-            new_seqs.sort(key=lambda s: s.prompt_tokens)   # stable: equal prompts keep arrival order
-        return new_seqs
+            admitted.sort(key=lambda s: s.prompt_tokens)   # stable: equal prompts keep arrival order
+        return admitted
 
     def _remove_finished(self) -> None:
         finished = [i for i, seq in enumerate(self.running_seqs)
@@ -126,5 +129,6 @@ class ModelHost:
         return self
 
     def __exit__(self, exc_type: Optional[Type[BaseException]], exc_val: Optional[BaseException],
-                 exc_tb: Optional[TracebackType]) -> None:
+                 exc_tb: Optional[TracebackType]) -> bool:
         self.stop()
+        return False   # an exception raised inside the with-block goes on to the caller

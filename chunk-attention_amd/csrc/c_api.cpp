@@ -3,6 +3,7 @@
 // include/chunk_attn_hip.h.
 #include "chunk_attn_hip.h"
 
+#include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -58,7 +59,51 @@ int guarded(F&& f) {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Named ranges in a profiler's marker trace (the reference brackets the same places with NVTX
+// ranges, kernel_cuda.cu:1334-1433).  The marker library is looked up at run time, only when
+// ca_set_markers asks for it: the shared library does not depend on it.
+struct Markers {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+    bool on = false;
+};
+Markers g_markers;
+
+struct Range {
+    bool open;
+    explicit Range(const char* name) : open(g_markers.on) {
+        if (open) g_markers.push(name);
+    }
+    ~Range() {
+        if (open) g_markers.pop();
+    }
+    Range(const Range&) = delete;
+    Range& operator=(const Range&) = delete;
+};
+
 }  // namespace
+
+int ca_set_markers(int enable) {
+    if (!enable) {
+        g_markers.on = false;
+        return CA_OK;
+    }
+    if (!g_markers.push) {
+        void* lib = nullptr;
+        for (const char* name : { "librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so" }) {
+            lib = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+            if (lib) break;
+        }
+        if (!lib) return fail(CA_ERR_STATE, "no marker library (roctx) could be loaded");
+        auto push = reinterpret_cast<int (*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+        auto pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+        if (!push || !pop) return fail(CA_ERR_STATE, "the marker library lacks roctxRangePushA / roctxRangePop");
+        g_markers.push = push;
+        g_markers.pop = pop;
+    }
+    g_markers.on = true;
+    return CA_OK;
+}
 
 // ---- kernel context ------------------------------------------------------------------------
 
@@ -437,6 +482,7 @@ void ca_ctx_destroy(ca_ctx* c) {
 int ca_refresh_kernel_context(ca_ctx* c, const ca_chunk_row* rows, int n_rows, int n_seqs,
                               void* stream) {
     if (!c || n_rows < 0 || n_seqs < 0 || (n_rows > 0 && !rows)) return fail(CA_ERR_INVALID, "bad argument");
+    Range range("ca_refresh_kernel_context");
     return guarded([&]() -> int {
         static_assert(sizeof(ca_chunk_row) == sizeof(ca::ChunkRow), "row layouts must agree");
         for (int i = 0; i < n_rows; i++) {
@@ -465,6 +511,7 @@ int ca_ctx_roll_tails(ca_ctx* c, const int32_t* seq_idx, const int32_t* new_slot
     for (int i = 0; i < n; i++) {
         if (new_slots[i] < 0 || new_slots[i] >= c->max_chunks) return fail(CA_ERR_INVALID, "slot outside the pool");
     }
+    Range range("ca_ctx_roll_tails");
     return guarded([&]() -> int {
         try {
             ca::roll_tails(&c->plan, c->C, plan_params(c, c->partition), c->delta_tokens, seq_idx, new_slots, n);
@@ -482,6 +529,15 @@ int ca_ctx_roll_tails(ca_ctx* c, const int32_t* seq_idx, const int32_t* new_slot
         c->delta_tokens = 0;
         c->valid = true;
         return CA_OK;
+    });
+}
+
+int ca_ctx_read_probe(ca_ctx* c, const void* dev, size_t bytes, void* stream) {
+    if (!c || !dev || bytes < 16 || (reinterpret_cast<uintptr_t>(dev) & 15)) return fail(CA_ERR_INVALID, "bad argument");
+    return guarded([&]() -> int {
+        float* sink = ca::scratch_ptr(c->device);
+        if (!sink) return fail(CA_ERR_STATE, "the static scratch buffer was not set up on this device");
+        return launch_rc(ca::launch_read_probe(dev, bytes, c->n_cus, sink, static_cast<hipStream_t>(stream)), "read probe");
     });
 }
 
@@ -504,6 +560,7 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
     if (int rc = check_attention_shape(c)) return rc;
     if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
     if (n_seqs == 0) return CA_OK;
+    Range range("ca_attention");
     return guarded([&]() -> int {
         hipStream_t st = static_cast<hipStream_t>(stream);
         if (partition != c->partition || c->schedule != c->plan_schedule) {
@@ -624,6 +681,7 @@ int ca_append_kv(ca_ctx* c, const void* k, const void* v, int n_seqs, void* stre
             return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
         }
     }
+    Range range("ca_append_kv");
     const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
     return launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
                                        reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),

@@ -56,6 +56,10 @@ int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st);
 // `st`.  For the table upload: a copy-engine transfer in the middle of a decode step costs the
 // stream several microseconds of hand-over between queues, a small kernel does not.
 int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream_t st);
+// Measurement aid: one workgroup per compute unit reads `bytes` of device memory (from a
+// 16-byte aligned address) with non-temporal 16-byte loads and keeps nothing; `sink` is 4
+// writable bytes of device memory.
+int launch_read_probe(const void* dev, size_t bytes, int n_cus, void* sink, hipStream_t st);
 int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32_t* tail_slot,
                   const int32_t* tail_fill, int n_seqs, hipStream_t st);
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,

@@ -1175,6 +1175,30 @@ __global__ __launch_bounds__(WG) void upload_kernel(uint4* __restrict__ dst, con
 // ---------------------------------------------------------------------------------------
 // K/V row writes.  One thread moves one piece (16 bytes when d_head allows, else 2) of K and V.
 // ---------------------------------------------------------------------------------------
+// Measurement aid: reads n16 16-byte units and keeps nothing.  Workgroup b, thread t reads unit
+// 256*b + t, then strides by the whole grid: at any moment the grid reads a few contiguous
+// megabytes, eight non-temporal loads per lane in flight.  What a read with no structure at
+// all reaches on this GPU: the yardstick beside the published peak.
+__global__ __launch_bounds__(WG) void read_probe_kernel(const uint4* __restrict__ p, size_t n16,
+                                                        uint32_t* __restrict__ sink) {
+    constexpr int U = 8;
+    const size_t stride = size_t(gridDim.x) * WG;
+    size_t i = size_t(blockIdx.x) * WG + threadIdx.x;
+    uint32_t acc = 0;
+    for (; i + (U - 1) * stride < n16; i += U * stride) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = nt_load16(p + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < U; u++) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n16; i += stride) {
+        const uint4 v = nt_load16(p + i);
+        acc += v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = acc;  // keeps the loads alive; practically never stores
+}
+
 template <typename T>
 __global__ __launch_bounds__(WG) void append_kernel(const T* __restrict__ k, const T* __restrict__ v,
                                                     T* __restrict__ kpool, T* __restrict__ vpool,
@@ -1341,6 +1365,14 @@ int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream
     const int n = static_cast<int>(bytes / 16);
     hipLaunchKernelGGL(upload_kernel, dim3((n + WG - 1) / WG), dim3(WG), 0, st, static_cast<uint4*>(dst_dev),
                        static_cast<const uint4*>(src_pinned), n);
+    CA_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_read_probe(const void* dev, size_t bytes, int n_cus, void* sink, hipStream_t st) {
+    if (bytes < 16 || !sink) return -1;
+    hipLaunchKernelGGL(read_probe_kernel, dim3(n_cus > 0 ? n_cus : 256), dim3(WG), 0, st,
+                       static_cast<const uint4*>(dev), bytes / 16, static_cast<uint32_t*>(sink));
     CA_LAUNCH_CHECK();
     return 0;
 }

@@ -25,6 +25,7 @@
 #ifndef CHUNK_ATTN_HIP_H
 #define CHUNK_ATTN_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -209,6 +210,18 @@ int ca_ctx_set_schedule(ca_ctx* ctx, int mode);
 int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
+
+/* Named ranges around table refreshes, table patches, attention calls and K/V appends in a
+ * profiler's marker trace (rocprofv3 --marker-trace), where the reference has NVTX ranges
+ * (kernel_cuda.cu:1334-1433).  Process-wide, off by default.  Enabling loads the roctx library
+ * at run time; CA_ERR_STATE when none is found. */
+int ca_set_markers(int enable);
+
+/* Measurement aid with no counterpart in the reference: one launch on `stream` that reads
+ * `bytes` of device memory at `dev` (16-byte aligned, at least 16 bytes) with plain streaming
+ * loads and keeps nothing: the read rate a kernel with no structure reaches on this GPU, for
+ * benchmarks to quote beside the published peak. */
+int ca_ctx_read_probe(ca_ctx* ctx, const void* dev, size_t bytes, void* stream);
 
 /* Numbers describing the current tables. */
 typedef struct ca_plan_info {

@@ -35,3 +35,21 @@ def test_device_entry_points_fail_loudly_without_a_gpu():
     h = ctypes.c_void_p()
     assert capi.load().ca_ctx_create(ctypes.byref(h), 0, 64, 64, None, None, 0, 1) == -1
     assert b"bad shape" in capi.load().ca_last_error()
+
+
+def test_markers_switch_on_and_off():
+    """Marker ranges are off by default; switching them on loads the roctx library at run time
+    (an error that says so where the image has none), and host-only calls still work inside them."""
+    import numpy as np
+    try:
+        capi.set_markers(True)
+    except capi.ChunkAttnError as e:
+        assert "marker library" in str(e)
+        return
+    try:
+        tree = capi.Tree(2, 16)
+        tree.add_seq([1, 2, 3])
+        rows = tree.get_chunks()
+        assert np.asarray(rows).shape[1] == 4
+    finally:
+        capi.set_markers(False)
