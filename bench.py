@@ -125,26 +125,39 @@ def cold_forward_us(attn, q, out, torch, reps=20, hints=(("default_policy", 0), 
 def plain_read_gbps(ctx, n_bytes, torch, reps=20):
     """What a read with no structure reaches on this GPU: the library's read probe (one
     workgroup per compute unit, non-temporal 16-byte loads, nothing kept) over a buffer of
-    n_bytes, repeated back to back (warm) and after a read of 1 GiB of other memory (cold), HIP
-    events around the launch; and over 2 GiB, where no cache helps and the launch's start and end
-    no longer weigh.  A yardstick beside the published peak, not a replacement for it."""
+    n_bytes under the decode launch's two protocols (warm: a back-to-back train between two HIP
+    events; cold: after a read of 1 GiB of other memory, events around the single launch), and
+    over 2 GiB, where no cache helps and the launch's start and end no longer weigh.  A yardstick
+    beside the published peak, not a replacement for it."""
     stream = torch.cuda.current_stream().cuda_stream
     flush = torch.zeros(1 << 27, dtype=torch.int64, device="cuda:0")
     res = {}
     for name, size, cold in (("warm", n_bytes, False), ("cold", n_bytes, True), ("2GiB", 2 << 30, False)):
         buf = torch.ones(max(size // 8, 2), dtype=torch.int64, device="cuda:0")
-        total = 0.0
-        for i in range(reps + 2):
-            if cold:
+        nb = buf.numel() * 8
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if cold:
+            total = 0.0
+            for i in range(reps + 2):
                 flush.sum()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                ctx.read_probe(buf.data_ptr(), nb, stream)
+                e1.record()
+                e1.synchronize()
+                if i >= 2:
+                    total += e0.elapsed_time(e1)
+            ms = total / reps
+        else:
+            n = reps if size <= (1 << 30) else 5
+            for _ in range(2):
+                ctx.read_probe(buf.data_ptr(), nb, stream)
             e0.record()
-            ctx.read_probe(buf.data_ptr(), buf.numel() * 8, stream)
+            for _ in range(n):
+                ctx.read_probe(buf.data_ptr(), nb, stream)
             e1.record()
             e1.synchronize()
-            if i >= 2:
-                total += e0.elapsed_time(e1)
-        res[name] = round(buf.numel() * 8 / (total * 1e-3 / reps) / 1e9, 1)
+            ms = e0.elapsed_time(e1) / n
+        res[name] = round(nb / (ms * 1e-3) / 1e9, 1)
         del buf
     del flush
     return res
@@ -447,6 +460,8 @@ def main() -> int:
                     help="also time the layer operators around the attention call (rms_norm, fused_add_rms_norm and "
                          "rotary_embedding on a prefill-sized batch): outside the metric, off by default")
     ap.add_argument("--no-pybind", action="store_true", help="skip timing the forward through the pybind11 class")
+    ap.add_argument("--markers", action="store_true",
+                    help="named roctx ranges around refreshes, patches, attention calls and appends (for rocprofv3 --marker-trace)")
     ap.add_argument("--seg-chunks", type=int, default=0)
     ap.add_argument("--stream-chunks", type=int, default=0)
     ap.add_argument("--stream-hint", type=int, default=0, help="non-temporal loads of private chunks: 0 by working-set size (default), 1 always, 2 never")
@@ -478,6 +493,8 @@ def main() -> int:
         print(json.dumps({"calibrate_copy_MiB": args.calibrate_copy, "copies": 20, "bytes_read_per_copy": n, "bytes_written_per_copy": n}))
         return 0
 
+    if args.markers:
+        capi.set_markers(True)
     w = synth.baseline_config(args.config, args.fraction)
     attn = build_cache(w, torch, capi, args.seed)
     if args.seg_chunks or args.stream_chunks:

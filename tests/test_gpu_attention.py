@@ -316,6 +316,24 @@ def test_negative_delta_tokens_is_rejected():
         attn.ctx.set_timing(7)
 
 
+def test_read_probe_reads_and_checks_its_arguments():
+    """The bench's yardstick launch: runs over aligned buffers of any length that holds one
+    16-byte unit, leaves the buffer alone, and rejects what it cannot read."""
+    w = synth.prefix_workload("rp", 2, 64, 64, 10, n_heads=2)
+    attn, _ = load_workload(w)
+    buf = torch.arange(1 << 18, dtype=torch.int64, device=dev())
+    before = buf.clone()
+    st = torch.cuda.current_stream().cuda_stream
+    for n_bytes in (16, 4096 + 16, buf.numel() * 8):
+        attn.ctx.read_probe(buf.data_ptr(), n_bytes, st)
+    torch.cuda.synchronize()
+    assert torch.equal(buf, before)
+    for ptr, n_bytes in ((buf.data_ptr() + 8, 64), (buf.data_ptr(), 8), (0, 64)):
+        with pytest.raises(capi.ChunkAttnError) as e:
+            attn.ctx.read_probe(ptr, n_bytes, st)
+        assert e.value.code == -1
+
+
 @pytest.mark.parametrize("c", [32, 64, 128])
 def test_repeated_forwards_are_bit_identical(c):
     """The default schedule merges partial rows in a fixed order, so a forward is a pure function
