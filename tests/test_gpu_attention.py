@@ -316,6 +316,27 @@ def test_negative_delta_tokens_is_rejected():
         attn.ctx.set_timing(7)
 
 
+def test_marker_ranges_do_not_change_results():
+    """roctx ranges around the C-ABI calls are bookkeeping on the host only."""
+    w = synth.prefix_workload("mk", 5, 64, 130, 70, n_heads=2)
+    attn, _ = load_workload(w)
+    q = to_dev(w.q())
+    base = attn.forward(q).clone()
+    try:
+        capi.set_markers(True)
+    except capi.ChunkAttnError as e:
+        assert "marker library" in str(e)
+        return
+    try:
+        attn.refresh_kernel_context(True)
+        k, v = w.append_kv(0)
+        assert torch.equal(attn.forward(q), base)
+        attn.append_token(w.append_tokens(0), to_dev(k), to_dev(v))
+        assert_close(attn.forward(q), oracle_output(attn, w.q()))
+    finally:
+        capi.set_markers(False)
+
+
 def test_read_probe_reads_and_checks_its_arguments():
     """The bench's yardstick launch: runs over aligned buffers of any length that holds one
     16-byte unit, leaves the buffer alone, and rejects what it cannot read."""
