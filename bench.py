@@ -122,9 +122,9 @@ def cold_forward_us(attn, q, out, torch, reps=20, hints=(("default_policy", 0), 
     return res
 
 
-def plain_read_gbps(ctx, n_bytes, torch, reps=20):
-    """What a read with no structure reaches on this GPU: the library's read probe (one
-    workgroup per compute unit, non-temporal 16-byte loads, nothing kept) over a buffer of
+def plain_read_gbps(ctx, n_bytes, torch, reps=20, wgs_per_cu=2):
+    """What a read with no structure reaches on this GPU: the library's read probe (wgs_per_cu
+    workgroups per compute unit, non-temporal 16-byte loads, nothing kept) over a buffer of
     n_bytes under the decode launch's two protocols (warm: a back-to-back train between two HIP
     events; cold: after a read of 1 GiB of other memory, events around the single launch), and
     over 2 GiB, where no cache helps and the launch's start and end no longer weigh.  A yardstick
@@ -141,7 +141,7 @@ def plain_read_gbps(ctx, n_bytes, torch, reps=20):
             for i in range(reps + 2):
                 flush.sum()
                 e0.record()
-                ctx.read_probe(buf.data_ptr(), nb, stream)
+                ctx.bench_read_probe(buf.data_ptr(), nb, wgs_per_cu, stream)
                 e1.record()
                 e1.synchronize()
                 if i >= 2:
@@ -150,10 +150,10 @@ def plain_read_gbps(ctx, n_bytes, torch, reps=20):
         else:
             n = reps if size <= (1 << 30) else 5
             for _ in range(2):
-                ctx.read_probe(buf.data_ptr(), nb, stream)
+                ctx.bench_read_probe(buf.data_ptr(), nb, wgs_per_cu, stream)
             e0.record()
             for _ in range(n):
-                ctx.read_probe(buf.data_ptr(), nb, stream)
+                ctx.bench_read_probe(buf.data_ptr(), nb, wgs_per_cu, stream)
             e1.record()
             e1.synchronize()
             ms = e0.elapsed_time(e1) / n
@@ -239,21 +239,19 @@ def pybind_cache(w, torch, seed, extra_chunks_per_seq=1):
     return attn
 
 
-def decode_launch_us(attn, q, out, steps, torch, mode=3):
-    """Average duration of the decode launch (mode 3), or of its sequence-first workgroups alone
-    (mode 4): a back-to-back train of that launch between two HIP events on the launch stream
-    (events around every single launch add 2-3 us each)."""
+def decode_launch_us(attn, q, out, steps, torch, what=0):
+    """Average duration of the decode launch (what 0), or of its sequence-first workgroups alone
+    (what 1): a back-to-back train of that launch between two HIP events on the launch stream
+    (events around every single launch add 2-3 us each).  `out` is left incomplete."""
     stream = torch.cuda.current_stream().cuda_stream
-    attn.ctx.set_timing(mode)
     for _ in range(5):
-        attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], 0, stream)
+        attn.ctx.bench_decode_launch(q.data_ptr(), out.data_ptr(), q.shape[0], what, stream)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(steps):
-        attn.ctx.attention(q.data_ptr(), out.data_ptr(), q.shape[0], 0, stream)
+        attn.ctx.bench_decode_launch(q.data_ptr(), out.data_ptr(), q.shape[0], what, stream)
     e1.record()
     e1.synchronize()
-    attn.ctx.set_timing(0)
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
@@ -506,7 +504,8 @@ def main() -> int:
     out = torch.empty_like(q)
 
     ms = time_forward(attn, q, out, args.steps, args.warmup, torch)
-    decode_ms = decode_launch_us(attn, q, out, min(args.steps, 200), torch) * 1e-3
+    scratch_out = torch.empty_like(q)   # the launch-only measurements leave their output incomplete
+    decode_ms = decode_launch_us(attn, q, scratch_out, min(args.steps, 200), torch) * 1e-3
     merge_ms = max(ms - decode_ms, 0.0)  # the step is the two launches back to back
     ph = phase_times(attn, q, out, min(args.steps, 50), torch, 2)
     info = attn.ctx.plan_info()
@@ -520,7 +519,7 @@ def main() -> int:
     decode_bytes = stream_bytes + shared_bytes + qo_bytes // 2
     achieved = decode_bytes / (decode_ms * 1e-3) / 1e9 if decode_ms > 0 else 0.0
     traffic, traffic_note = measured_traffic(w.name, info)
-    stream_us = decode_launch_us(attn, q, out, min(args.steps, 200), torch, mode=4) if info.n_stream_items else 0.0
+    stream_us = decode_launch_us(attn, q, scratch_out, min(args.steps, 200), torch, what=1) if info.n_stream_items else 0.0
     train_gbps = stream_bytes / (stream_us * 1e-6) / 1e9 if stream_us > 0 else 0.0
     stream_gbps = stream_bytes / (ph["stream_ms"] * 1e-3) / 1e9 if ph["stream_ms"] > 0 else 0.0
 

@@ -63,6 +63,8 @@ SIGNATURES = {
                                           ctypes.c_int, ctypes.c_void_p]),
     "ca_append_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                     ctypes.c_void_p]),
+    "ca_decode_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_rotary_embedding": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                            ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
@@ -77,6 +79,7 @@ SIGNATURES = {
     "ca_scatter_kv": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "ca_copy_chunks": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_put_kv_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, c_i32_p,
                                       ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
@@ -84,7 +87,10 @@ SIGNATURES = {
     "ca_ctx_set_stream_hint": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_set_markers": (ctypes.c_int, [ctypes.c_int]),
     "ca_ctx_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
-    "ca_ctx_read_probe": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "ca_bench_decode_launch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                              ctypes.c_int, ctypes.c_void_p]),
+    "ca_bench_read_probe": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                                           ctypes.c_void_p]),
     "ca_ctx_read_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_int64), ctypes.c_int]),
@@ -517,6 +523,10 @@ class KernelContext:
     def append_kv(self, k_ptr: int, v_ptr: int, n_seqs: int, stream: int = 0) -> None:
         _check(self._lib.ca_append_kv(self._h, k_ptr, v_ptr, n_seqs, stream))
 
+    def decode_step(self, q_ptr: int, k_ptr: int, v_ptr: int, out_ptr: int, n_seqs: int, stream: int = 0) -> None:
+        """append_kv + delta_tokens += 1 + attention (partition 0) in one call, one launch fewer."""
+        _check(self._lib.ca_decode_step(self._h, q_ptr, k_ptr, v_ptr, out_ptr, n_seqs, stream))
+
     def rope_append_kv(self, positions_ptr: int, q_ptr: int, k_ptr: int, v_ptr: int, cache_ptr: int,
                        max_position: int, rot_dim: int, is_neox: bool, n_seqs: int, stream: int = 0) -> None:
         _check(self._lib.ca_rope_append_kv(self._h, positions_ptr or None, q_ptr, k_ptr, v_ptr, cache_ptr,
@@ -536,6 +546,13 @@ class KernelContext:
     def copy_chunk(self, src_slot: int, dst_slot: int, stream: int = 0) -> None:
         _check(self._lib.ca_copy_chunk(self._h, src_slot, dst_slot, stream))
 
+    def copy_chunks(self, pairs: Sequence[Tuple[int, int]], stream: int = 0) -> None:
+        """Chunk pairs[i][0] copied onto chunk pairs[i][1], all pairs in one launch."""
+        if not pairs:
+            return
+        arr, ptr = _i32([x for p in pairs for x in p])
+        _check(self._lib.ca_copy_chunks(self._h, ptr, len(pairs), stream))
+
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
 
@@ -548,13 +565,17 @@ class KernelContext:
         _check(self._lib.ca_ctx_set_schedule(self._h, int(mode)))
 
     def set_timing(self, mode: int) -> None:
-        """0 off, 1 time the fused launch, 2 run and time the three phases separately, 3 / 4 issue only
-        the decode launch / only its sequence-first workgroups (for timing a train of them)."""
+        """0 off, 1 time the forward's launches, 2 run and time the three phases separately."""
         _check(self._lib.ca_ctx_set_timing(self._h, int(mode)))
 
-    def read_probe(self, dev_ptr: int, n_bytes: int, stream: int = 0) -> None:
+    def bench_decode_launch(self, q_ptr: int, out_ptr: int, n_seqs: int, what: int = 0, stream: int = 0) -> None:
+        """Measurement aid: the decode launch alone (0), its stream items alone (1) or its shared items
+        alone (2); the output is not complete afterwards."""
+        _check(self._lib.ca_bench_decode_launch(self._h, q_ptr, out_ptr, n_seqs, what, stream))
+
+    def bench_read_probe(self, dev_ptr: int, n_bytes: int, wgs_per_cu: int = 1, stream: int = 0) -> None:
         """Measurement aid: one launch that reads n_bytes of device memory and keeps nothing."""
-        _check(self._lib.ca_ctx_read_probe(self._h, dev_ptr, n_bytes, stream))
+        _check(self._lib.ca_bench_read_probe(self._h, dev_ptr, n_bytes, wgs_per_cu, stream))
 
     def read_timing(self, reset: bool = True) -> dict:
         """Accumulated per-phase milliseconds of the timed ca_attention calls."""
@@ -685,6 +706,23 @@ class Attention:
         self.ctx.delta_tokens = self.ctx.delta_tokens + 1
         return n_new
 
+    def decode_step(self, tokens: Sequence[int], q, k, v):
+        """append_token(tokens, k, v) followed by forward(q) as one call (same results, bit for bit):
+        the new K/V rows are written by the attention launch itself.  Returns the output."""
+        import torch
+        n = len(tokens)
+        if self.tree.n_seqs != n:
+            raise RuntimeError("num of seqs is not equal to num of tokens")
+        k = self._check_kv(k, n, "k")
+        v = self._check_kv(v, n, "v")
+        q = self._check_kv(q, n, "q")
+        self.reserve()
+        self.refresh_kernel_context()
+        out = torch.empty((n, self.n_heads, self.d_head), dtype=q.dtype, device=q.device)
+        self.ctx.decode_step(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), n, self._stream())
+        self.tree.append_token(tokens)  # reserve inside is a no-op now
+        return out
+
     def append_token_rotary(self, tokens: Sequence[int], q, k, v, cos_sin_cache, is_neox: bool = True,
                             positions=None) -> int:
         """append_token with the rotary embedding of the new rows folded in: q is rotated in
@@ -719,8 +757,7 @@ class Attention:
     def duplicate(self, seq_idx: int, copies: int) -> None:
         """Beam search: `copies` more sequences identical to seq_idx, right after it (reference
         attention.cpp:287-313); each owns a device copy of the tail chunk."""
-        for src, dst in self.tree.duplicate(seq_idx, copies):
-            self.ctx.copy_chunk(src, dst, self._stream())
+        self.ctx.copy_chunks(self.tree.duplicate(seq_idx, copies), self._stream())
         self.ctx.invalidate()
 
     def append_completion(self, seq_idx: int, tokens: Sequence[int], k, v) -> int:
@@ -732,8 +769,7 @@ class Attention:
         k = self._check_kv(k, n, "k")
         v = self._check_kv(v, n, "v")
         pairs, targets = self.tree.append_completion(seq_idx, tokens)
-        for src, dst in pairs:
-            self.ctx.copy_chunk(src, dst, self._stream())
+        self.ctx.copy_chunks(pairs, self._stream())
         self.ctx.put_kv_rows(k.data_ptr(), v.data_ptr(), targets, self._stream())   # same stream: after the copies
         self.ctx.invalidate()
         return seq_idx

@@ -198,6 +198,24 @@ std::vector<Chunk*> Attention::append_token_rotary(const std::vector<int>& token
     return fresh;
 }
 
+torch::Tensor Attention::decode_step(const std::vector<int>& tokens, torch::Tensor q, torch::Tensor k,
+                                     torch::Tensor v) {
+    if (tree_->tails().size() != tokens.size()) {
+        throw std::runtime_error("num of seqs is not equal to num of tokens");
+    }
+    const int n = static_cast<int>(tokens.size());
+    k = checked_kv(k, n, "k");
+    v = checked_kv(v, n, "v");
+    q = checked_kv(q, n, "q");
+    reserve_and_note();
+    refresh_kernel_context();
+    c10::DeviceGuard guard(t_options_.device());
+    torch::Tensor output = torch::empty({ q.size(0), n_heads_, d_head_ }, t_options_);
+    check(ca_decode_step(ctx_, q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), n, stream()));
+    tree_->append_token_ids(tokens);
+    return output;
+}
+
 torch::Tensor Attention::forward(torch::Tensor q, int partition) {
     if (!q.is_contiguous()) throw std::runtime_error("q is not contiguous");
     if (q.dim() != 3 || q.size(1) != n_heads_ || q.size(2) != d_head_) {
@@ -216,7 +234,17 @@ void Attention::duplicate(int seq_idx, int copies) {
     std::vector<std::pair<int, int>> pairs;
     tree_->duplicate(seq_idx, copies, &pairs);
     c10::DeviceGuard guard(t_options_.device());
-    for (const auto& [src, dst] : pairs) check(ca_copy_chunk(ctx_, src, dst, stream()));
+    copy_chunks(pairs);
+}
+
+void Attention::copy_chunks(const std::vector<std::pair<int, int>>& pairs) {
+    std::vector<int32_t> flat;
+    flat.reserve(2 * pairs.size());
+    for (const auto& [src, dst] : pairs) {
+        flat.push_back(src);
+        flat.push_back(dst);
+    }
+    check(ca_copy_chunks(ctx_, flat.data(), static_cast<int>(pairs.size()), stream()));
 }
 
 int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::Tensor k, torch::Tensor v) {
@@ -231,7 +259,7 @@ int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::T
     std::vector<PrefixTree::RowTarget> rows;
     tree_->append_completion(seq_idx, tokens, &pairs, &rows);
     c10::DeviceGuard guard(t_options_.device());
-    for (const auto& [src, dst] : pairs) check(ca_copy_chunk(ctx_, src, dst, stream()));
+    copy_chunks(pairs);  // one launch for every candidate's copy of the tail
     // row i of k/v is the new token of sequence seq_idx + i (same stream: after the copies)
     std::vector<int32_t> slot_row;
     for (const auto& r : rows) {

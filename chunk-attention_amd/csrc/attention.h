@@ -45,6 +45,11 @@ class Attention {
                                             torch::Tensor k, torch::Tensor v,
                                             torch::Tensor cos_sin_cache, bool is_neox = true,
                                             c10::optional<torch::Tensor> positions = c10::nullopt);
+    // One decode step: append_token(tokens, k, v) followed by forward(q), with the same results
+    // bit for bit, as one call: the attention launch writes the new K/V rows itself (one launch
+    // fewer per step).  q, k, v: [n_seqs, n_heads, d_head].  Returns the output.
+    torch::Tensor decode_step(const std::vector<int>& tokens, torch::Tensor q, torch::Tensor k,
+                              torch::Tensor v);
     void refresh_kernel_context(bool force = false);
     std::vector<Chunk*> reserve();
     void clear();
@@ -69,6 +74,7 @@ class Attention {
     void* stream() const;
     void check(int rc) const;
     torch::Tensor checked_kv(const torch::Tensor& t, int64_t rows, const char* name) const;
+    void copy_chunks(const std::vector<std::pair<int, int>>& pairs);  // (source slot, destination slot)
 
     int n_heads_, d_head_, chunk_size_, memory_mb_;
     bool share_prefix_;

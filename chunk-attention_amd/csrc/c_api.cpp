@@ -7,9 +7,11 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <exception>
+#include <mutex>
 #include <new>
 #include <stdexcept>
 #include <string>
@@ -62,16 +64,19 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // Named ranges in a profiler's marker trace (the reference brackets the same places with NVTX
 // ranges, kernel_cuda.cu:1334-1433).  The marker library is looked up at run time, only when
 // ca_set_markers asks for it: the shared library does not depend on it.
+// Process-wide: `on` is read by every entry point of every thread, the function pointers are
+// written once (under the mutex) before `on` is first set.
 struct Markers {
+    std::mutex load;  // serialises the lookup of the marker library
     int (*push)(const char*) = nullptr;
     int (*pop)() = nullptr;
-    bool on = false;
+    std::atomic<bool> on{ false };
 };
 Markers g_markers;
 
 struct Range {
     bool open;
-    explicit Range(const char* name) : open(g_markers.on) {
+    explicit Range(const char* name) : open(g_markers.on.load(std::memory_order_acquire)) {
         if (open) g_markers.push(name);
     }
     ~Range() {
@@ -85,9 +90,10 @@ struct Range {
 
 int ca_set_markers(int enable) {
     if (!enable) {
-        g_markers.on = false;
+        g_markers.on.store(false, std::memory_order_release);
         return CA_OK;
     }
+    std::lock_guard<std::mutex> lock(g_markers.load);
     if (!g_markers.push) {
         void* lib = nullptr;
         for (const char* name : { "librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so" }) {
@@ -101,7 +107,7 @@ int ca_set_markers(int enable) {
         g_markers.push = push;
         g_markers.pop = pop;
     }
-    g_markers.on = true;
+    g_markers.on.store(true, std::memory_order_release);
     return CA_OK;
 }
 
@@ -162,7 +168,7 @@ struct ca_ctx {
     std::vector<void*> retired_host;  // pinned staging buffers that were outgrown
 
     // optional timing: events recorded on the caller's stream around the launches.
-    // 1: the fused launch; 2: forward run as three timed launches (chunk-first, sequence-first, merge)
+    // 1: the forward as it runs; 2: forward run as three timed launches (chunk-first, sequence-first, merge)
     int timing = 0;
     hipEvent_t ev[4] = { nullptr, nullptr, nullptr, nullptr };
     bool ev_pending = false;
@@ -205,6 +211,7 @@ ca::LaunchArgs launch_args(const ca_ctx* c, const void* q, void* out) {
     a.d = c->d;
     a.scale_log2 = 1.4426950408889634f / std::sqrt(static_cast<float>(c->d));
     a.stream_per_wave = c->plan.stream_per_wave;
+    a.shared_narrow = c->plan.shared_narrow;
     // 256 MiB of Infinity Cache on this part.  A forward that attends more than that cannot find
     // its K/V there again on the next step, and plain loads top out near 6.3 TB/s against
     // 7.2 TB/s for loads with the non-temporal hint (measured with a bare read kernel): stream
@@ -532,15 +539,6 @@ int ca_ctx_roll_tails(ca_ctx* c, const int32_t* seq_idx, const int32_t* new_slot
     });
 }
 
-int ca_ctx_read_probe(ca_ctx* c, const void* dev, size_t bytes, void* stream) {
-    if (!c || !dev || bytes < 16 || (reinterpret_cast<uintptr_t>(dev) & 15)) return fail(CA_ERR_INVALID, "bad argument");
-    return guarded([&]() -> int {
-        float* sink = ca::scratch_ptr(c->device);
-        if (!sink) return fail(CA_ERR_STATE, "the static scratch buffer was not set up on this device");
-        return launch_rc(ca::launch_read_probe(dev, bytes, c->n_cus, sink, static_cast<hipStream_t>(stream)), "read probe");
-    });
-}
-
 int ca_ctx_valid(const ca_ctx* c) { return c && c->valid; }
 void ca_ctx_invalidate(ca_ctx* c) {
     if (c) c->valid = false;
@@ -567,16 +565,6 @@ int ca_attention(ca_ctx* c, const void* q, void* out, int n_seqs, int partition,
             if (int rc = build_and_upload(c, partition, st)) return rc;
         }
         if (!c->timing) return run_fused(c, q, out, st);
-        if (c->timing == 3) {
-            // measurement aid: only the decode launch, so that a caller can time a train of them
-            const ca::LaunchArgs a3 = launch_args(c, q, out);
-            return launch_rc(ca::launch_decode(a3, static_cast<int>(c->plan.shared_items.size()),
-                                               static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
-        }
-        if (c->timing == 4) {
-            // measurement aid: only the sequence-first workgroups (the stream items)
-            return run_stream(c, q, out, st);
-        }
         if (int rc = collect_timing(c)) return rc;
         CA_HIP(hipEventRecord(c->ev[0], st));
         if (c->timing == 1 && c->schedule == 0) {
@@ -630,9 +618,50 @@ int ca_attention_noalloc(ca_ctx* c, const void* q, void* out, int n_seqs, void* 
     return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
 }
 
+static_assert(CA_NOALLOC_SCRATCH_BYTES == ca::kScratchBytes, "the header's scratch size and the kernels' must agree");
+
+int ca_decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs, void* stream) {
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
+    if (n_seqs > 0 && (!out || !k || !v)) return fail(CA_ERR_INVALID, "null device pointer");
+    if (n_seqs == 0) return CA_OK;
+    for (int s = 0; s < n_seqs; s++) {
+        if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
+            return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
+        }
+    }
+    Range range("ca_decode_step");
+    return guarded([&]() -> int {
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (c->partition != 0 || c->schedule != c->plan_schedule) {
+            if (int rc = build_and_upload(c, 0, st)) return rc;
+        }
+        if (c->schedule == 0 && c->plan.tails_streamed) {
+            // one launch appends and attends: the workgroup that streams a sequence's last chunk
+            // takes the new row from k / v and writes it into the pool on the way
+            c->delta_tokens += 1;
+            ca::LaunchArgs a = launch_args(c, q, out);
+            a.k_new = k;
+            a.v_new = v;
+            int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                                 static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
+            if (rc == CA_OK) rc = run_merge(c, out, st);
+            if (rc != CA_OK) c->delta_tokens -= 1;
+            return rc;
+        }
+        // last chunks attended chunk-first, or the single-launch schedule: append, then attend
+        const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+        if (int rc = launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
+                                                 reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
+                                                 n_seqs, st), "append launch")) return rc;
+        c->delta_tokens += 1;
+        return run_fused(c, q, out, st);
+    });
+}
+
 int ca_ctx_set_timing(ca_ctx* c, int enable) {
     if (!c) return fail(CA_ERR_INVALID, "null context");
-    if (enable < 0 || enable > 4) return fail(CA_ERR_INVALID, "timing mode must be 0, 1, 2, 3 or 4");
+    if (enable < 0 || enable > 2) return fail(CA_ERR_INVALID, "timing mode must be 0, 1 or 2");
     if (enable && !c->ev[0]) {
         for (int i = 0; i < 4; i++) CA_HIP(hipEventCreate(&c->ev[i]));
     }
@@ -798,15 +827,31 @@ int ca_scatter_kv(ca_ctx* c, const void* k, const void* v, int n_tokens, int tok
                                         static_cast<hipStream_t>(stream)), "scatter launch");
 }
 
-int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
-    if (!c || src_slot < 0 || dst_slot < 0 || src_slot >= c->max_chunks || dst_slot >= c->max_chunks) {
-        return fail(CA_ERR_INVALID, "slot outside the pool");
+int ca_copy_chunks(ca_ctx* c, const int32_t* src_dst, int n_pairs, void* stream) {
+    if (!c || n_pairs < 0) return fail(CA_ERR_INVALID, "bad argument");
+    if (n_pairs == 0) return CA_OK;
+    if (!src_dst) return fail(CA_ERR_INVALID, "null pointer");
+    for (int i = 0; i < n_pairs; i++) {
+        const int src = src_dst[2 * i], dst = src_dst[2 * i + 1];
+        if (src < 0 || dst < 0 || src >= c->max_chunks || dst >= c->max_chunks) {
+            return fail(CA_ERR_INVALID, "slot outside the pool");
+        }
+        if (src == dst) return fail(CA_ERR_INVALID, "a chunk cannot be copied onto itself");
+        for (int j = 0; j < n_pairs; j++) {
+            // one launch: a chunk written by one pair must not be read or written by another
+            if (j != i && (src_dst[2 * j] == dst || (j < i && src_dst[2 * j + 1] == dst))) {
+                return fail(CA_ERR_INVALID, "copy pairs overlap: a destination is also a source or written twice");
+            }
+        }
     }
-    const size_t bytes = size_t(c->H) * c->C * c->d * 2;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    CA_HIP(hipMemcpyAsync(static_cast<char*>(c->k_pool) + bytes * dst_slot, static_cast<char*>(c->k_pool) + bytes * src_slot, bytes, hipMemcpyDeviceToDevice, st));
-    CA_HIP(hipMemcpyAsync(static_cast<char*>(c->v_pool) + bytes * dst_slot, static_cast<char*>(c->v_pool) + bytes * src_slot, bytes, hipMemcpyDeviceToDevice, st));
-    return CA_OK;
+    if ((size_t(c->H) * c->C * c->d * 2) % 16 != 0) return fail(CA_ERR_INVALID, "chunk size in bytes must be a multiple of 16");
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    return launch_rc(ca::launch_copy_chunks(a, src_dst, n_pairs, static_cast<hipStream_t>(stream)), "chunk copy launch");
+}
+
+int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
+    const int32_t pair[2] = { src_slot, dst_slot };
+    return ca_copy_chunks(c, pair, 1, stream);
 }
 
 int ca_put_kv_rows(ca_ctx* c, const void* k, const void* v, int n_rows, const int32_t* slot_row, void* stream) {
@@ -938,6 +983,33 @@ int ca_ctx_read_partials_raw(ca_ctx* c, float* out, int64_t n_floats, void* stre
     if (n > 0) CA_HIP(hipMemcpyAsync(out, c->part, size_t(n) * 4, hipMemcpyDeviceToHost, st));
     CA_HIP(hipStreamSynchronize(st));
     return CA_OK;
+}
+
+// ---- measurement aids (not for callers) ------------------------------------------------------
+
+int ca_bench_decode_launch(ca_ctx* c, const void* q, void* out, int n_seqs, int what, void* stream) {
+    if (what < 0 || what > 2) return fail(CA_ERR_INVALID, "what must be 0 (whole decode launch), 1 (stream items) or 2 (shared items)");
+    if (int rc = check_ready(c, q, n_seqs)) return rc;
+    if (int rc = check_attention_shape(c)) return rc;
+    if (n_seqs > 0 && !out) return fail(CA_ERR_INVALID, "null device pointer");
+    if (n_seqs == 0) return CA_OK;
+    if (c->partition != 0 || c->schedule != 0 || c->plan_schedule != 0) {
+        return fail(CA_ERR_STATE, "the tables were built for another partition or schedule");
+    }
+    const ca::LaunchArgs a = launch_args(c, q, out);
+    const int n_shared = what == 1 ? 0 : static_cast<int>(c->plan.shared_items.size());
+    const int n_stream = what == 2 ? 0 : static_cast<int>(c->plan.stream_items.size());
+    return launch_rc(ca::launch_decode(a, n_shared, n_stream, false, static_cast<hipStream_t>(stream)), "decode launch");
+}
+
+int ca_bench_read_probe(ca_ctx* c, const void* dev, size_t bytes, int wgs_per_cu, void* stream) {
+    if (!c || !dev || bytes < 16 || (reinterpret_cast<uintptr_t>(dev) & 15)) return fail(CA_ERR_INVALID, "bad argument");
+    if (wgs_per_cu < 1 || wgs_per_cu > 8) return fail(CA_ERR_INVALID, "wgs_per_cu must be 1 .. 8");
+    return guarded([&]() -> int {
+        void* sink = ca::probe_sink_ptr(c->device);
+        if (!sink) return fail(CA_ERR_STATE, "the static device buffers were not set up on this device");
+        return launch_rc(ca::launch_read_probe(dev, bytes, c->n_cus * wgs_per_cu, sink, static_cast<hipStream_t>(stream)), "read probe");
+    });
 }
 
 // ---- host-only table builder ---------------------------------------------------------------

@@ -34,6 +34,13 @@ struct LaunchArgs {
     // Every wave of a stream workgroup takes a stream item of its own (four consecutive items per
     // workgroup): set by the plan when there are many short runs.  Not with fuse_merge.
     bool stream_per_wave = false;
+    // No shared item of the work list covers more than 16 sequences and none is wide: the launch
+    // can take the form of the kernel without the 32-row and wide matrix-core paths.
+    bool shared_narrow = false;
+    // Fused decode step: rows [n_seqs, H, 128] of the token appended by this launch (delta_tokens
+    // already counts it).  Needs a work list in which every sequence's last chunk is streamed.
+    const void* k_new = nullptr;
+    const void* v_new = nullptr;
 };
 
 // Static device scratch for the entry point that allocates nothing: a file-scope __device__
@@ -43,6 +50,9 @@ struct LaunchArgs {
 constexpr size_t kScratchBytes = size_t(32) << 20;
 int scratch_setup(int device);   // 0 or a positive hipError_t
 float* scratch_ptr(int device);
+// 16 bytes of device memory of its own for the read probe's never-taken store (resolved by
+// scratch_setup as well)
+void* probe_sink_ptr(int device);
 
 // All return 0, -1 for an unsupported shape, or a positive hipError_t.
 // One launch over the first n_shared_items shared items and the first n_stream_items stream
@@ -56,14 +66,17 @@ int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st);
 // `st`.  For the table upload: a copy-engine transfer in the middle of a decode step costs the
 // stream several microseconds of hand-over between queues, a small kernel does not.
 int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream_t st);
-// Measurement aid: one workgroup per compute unit reads `bytes` of device memory (from a
-// 16-byte aligned address) with non-temporal 16-byte loads and keeps nothing; `sink` is 4
-// writable bytes of device memory.
-int launch_read_probe(const void* dev, size_t bytes, int n_cus, void* sink, hipStream_t st);
+// Measurement aid: n_wgs workgroups read `bytes` of device memory (from a 16-byte aligned
+// address) with non-temporal 16-byte loads and keep nothing; `sink` is 4 writable bytes of
+// device memory.
+int launch_read_probe(const void* dev, size_t bytes, int n_wgs, void* sink, hipStream_t st);
 int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32_t* tail_slot,
                   const int32_t* tail_fill, int n_seqs, hipStream_t st);
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,
                    const int32_t* slots, int n_slots, hipStream_t st);
+// chunk src_dst[2i] of both pools copied onto chunk src_dst[2i+1], i < n_pairs (host array), one
+// launch per 64 pairs; the pairs must not overlap
+int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, hipStream_t st);
 // rows i < n of k/v ([n, H, d]) to row slot_row[2i+1] of chunk slot_row[2i] (host array)
 int launch_put_rows(const LaunchArgs& a, const void* k, const void* v, const int32_t* slot_row, int n,
                     hipStream_t st);

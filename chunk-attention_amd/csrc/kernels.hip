@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <mutex>
 #include <type_traits>
 
 #include "kernels.h"
@@ -207,6 +208,10 @@ struct DecodeArgs {
     int n_stream_items;   // stream items in the list
     int stream_per_wave;  // 1: every wave of a stream workgroup takes an item of its own (needs fuse_merge 0)
     int stream_nt;   // 1: private chunks are read with the non-temporal hint (see LaunchArgs)
+    // Fused decode step (stream_path<.., APPEND>): the newest token of every sequence, [n_seqs, H, D].
+    // delta_tokens already counts it; its row in the pool is written by the workgroup that attends it.
+    const half_t* k_new;
+    const half_t* v_new;
 };
 
 // Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
@@ -261,15 +266,15 @@ constexpr int VPITCH = D + 16;  // halves per LDS row of a V block: 288 B puts t
                                 // four consecutive token rows into four different bank groups,
                                 // and rows stay 16-byte aligned for whole-vector writes
 constexpr int OPITCH = D + 4;  // floats per row of the cross-wave accumulation buffer
-constexpr int MB = 2;          // 16-row blocks per shared item
-constexpr int MROWS = 16 * MB;
+// MBT: 16-row blocks per shared item (2: items of up to 32 sequences, 1: up to 16)
+template <int MBT>
 struct SharedPathLds {
     half_t v[NW][16 * VPITCH];
-    float o[MROWS * OPITCH];
-    float m[NW][MROWS];
-    float l[NW][MROWS];
-    int last[MROWS];
-    int row[MROWS];  // partial row of each covered sequence
+    float o[16 * MBT * OPITCH];
+    float m[NW][16 * MBT];
+    float l[NW][16 * MBT];
+    int last[16 * MBT];
+    int row[16 * MBT];  // partial row of each covered sequence
 };
 struct StreamPathLds {
     float p[NW][64];
@@ -283,16 +288,31 @@ struct StreamPathLds {
 // 16-byte columns g and g+1) fall into sixteen different 16-byte bank groups.  (272 B, which only
 // separates the rows of one group, costs every such read a second pass: measured with the LDS
 // bank-conflict counter.)
-constexpr int WROWS = 4 * MROWS;  // sequences per wide item: 32 per wave
+constexpr int WROWS = 128;  // sequences per wide item: 32 per wave
 struct WidePathLds {
     half_t k[1][64 * VPITCH];
     half_t v[1][64 * VPITCH];
     int last[WROWS];
 };
-union __attribute__((aligned(16))) DecodeLds {
-    SharedPathLds sh;
+// The decode kernel exists in three forms, chosen on the host from what the work list holds, so
+// that launches without the wide matrix-core path are not held to its register and LDS budget
+// (two workgroups per compute unit) and run three per compute unit instead:
+//   kMixFull    every path;
+//   kMixStream  stream items only (nothing shared, or partition 2);
+//   kMixNarrow  stream items and shared items of at most 16 sequences, none wide.
+constexpr int kMixFull = 0, kMixStream = 1, kMixNarrow = 2;
+template <int MIX> union DecodeLds;
+template <> union __attribute__((aligned(16))) DecodeLds<kMixFull> {
+    SharedPathLds<2> sh;
     StreamPathLds st;
     WidePathLds wd;
+};
+template <> union __attribute__((aligned(16))) DecodeLds<kMixStream> {
+    StreamPathLds st;
+};
+template <> union __attribute__((aligned(16))) DecodeLds<kMixNarrow> {
+    SharedPathLds<1> sh;
+    StreamPathLds st;
 };
 
 // ---------------------------------------------------------------------------------------
@@ -304,7 +324,12 @@ union __attribute__((aligned(16))) DecodeLds {
 // ---------------------------------------------------------------------------------------
 // PER_WAVE: the wave works alone on its own item (all tiles, no cross-wave combine, no barrier):
 // the form for many short runs, where a workgroup per run would spend its life starting up.
-template <int C, bool PER_WAVE>
+// APPEND: the fused decode step.  The newest token of the sequence (position len - 1) has no row
+// in the pool yet: the wave whose tile holds that position takes the row from k_new / v_new
+// instead, and the 16 lanes that hold it store it into the pool.  Nobody else reads that row in
+// this launch (the last chunk of a sequence belongs to exactly one stream item), and the
+// arithmetic is that of a forward over a pool the row was appended to beforehand.
+template <int C, bool PER_WAVE, bool APPEND>
 __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, StreamPathLds& sm) {
     WorkItem it;  // header only: the inline slots are read from global memory where needed
@@ -401,6 +426,8 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
         // tokens of this tile: bounded by the sequence's end and by the item's last chunk (the
         // sequence may go on in another item)
         const int n_here = (it.n_chunks - t < CPT) ? it.n_chunks - t : CPT;
+        // the sequence ends inside this tile: the tile of its newest token
+        const bool tile_has_new = APPEND && valid <= n_here * C;
         valid = valid < n_here * C ? valid : n_here * C;
         size_t base[CPT];
 #pragma unroll
@@ -412,7 +439,8 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
         for (int sub = 0; sub < NSUB; sub++) {
             const int vsub = valid - sub * SUB;  // valid rows in this sub-tile
             if (vsub <= 0) break;
-            const bool masked = vsub < SUB;
+            const bool new_here = tile_has_new && vsub <= SUB;  // the newest token is row vsub - 1
+            const bool masked = vsub < SUB || new_here;
             // load i of the sub-tile: 1 KiB at offset (i % LPC) KiB of chunk i / LPC
             const uint4* kp[CPT];
             const uint4* vp[CPT];
@@ -435,11 +463,49 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
                 }
             } else {
                 // rows past the end of the sequence hold stale data: never read into the math
+                const int vmem = (APPEND && new_here) ? vsub - 1 : vsub;  // rows that the pool holds
 #pragma unroll
                 for (int i = 0; i < NL; i++) {
-                    const bool ok = 4 * i + g < vsub;
+                    const bool ok = 4 * i + g < vmem;
                     kr[i] = ok ? kp[i / LPC][64 * (i % LPC)] : make_uint4(0, 0, 0, 0);
                     vr[i] = ok ? vp[i / LPC][64 * (i % LPC)] : make_uint4(0, 0, 0, 0);
+                }
+                if constexpr (APPEND) {
+                    if (new_here) {
+                        // row vsub - 1 = 4 * i_new + g_new is the newest token: lanes (g_new, j) take
+                        // piece j of it from the caller's rows, as if it had been loaded from the
+                        // pool, and put it there
+                        const int i_new = (vsub - 1) >> 2;
+                        const bool mine = ((vsub - 1) & 3) == g;
+                        const size_t new_off = (size_t(seq) * H + h) * D;
+                        // K, then V: one row piece at a time keeps the register count down
+                        {
+                            const uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
+#pragma unroll
+                            for (int i = 0; i < NL; i++) {
+                                if (i == i_new && mine) kr[i] = kn;
+                            }
+                            uint4* kd = const_cast<uint4*>(kp[0]);
+#pragma unroll
+                            for (int cc = 1; cc < CPT; cc++) {
+                                if (i_new / LPC == cc) kd = const_cast<uint4*>(kp[cc]);
+                            }
+                            if (mine) kd[64 * (i_new % LPC)] = kn;
+                        }
+                        {
+                            const uint4 vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
+#pragma unroll
+                            for (int i = 0; i < NL; i++) {
+                                if (i == i_new && mine) vr[i] = vn;
+                            }
+                            uint4* vd = const_cast<uint4*>(vp[0]);
+#pragma unroll
+                            for (int cc = 1; cc < CPT; cc++) {
+                                if (i_new / LPC == cc) vd = const_cast<uint4*>(vp[cc]);
+                            }
+                            if (mine) vd[64 * (i_new % LPC)] = vn;
+                        }
+                    }
                 }
             }
             float sc[NL];
@@ -583,9 +649,10 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
 //   of the 16 x 128 V block through the LDS transpose read (lds_read_tr).
 // ---------------------------------------------------------------------------------------
-template <int C>
+template <int C, int MBT>
 __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
-                                            int h, SharedPathLds& sm) {
+                                            int h, SharedPathLds<MBT>& sm) {
+    constexpr int MB = MBT;  // 16-row blocks of the item
     WorkItem it;
     it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
     it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
@@ -601,7 +668,7 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     const int l = tid & 63, g = l >> 4, i = l & 15;
     const int slotv = preload_slots(gi, it.slot_first, it.n_chunks, slots, l);
     const int len = it.len0 + A.delta_tokens;
-    const bool two = it.n_rows > 16;  // second 16-row block in use (uniform)
+    const bool two = MB > 1 && it.n_rows > 16;  // second 16-row block in use (uniform)
     if (tid < it.n_rows) sm.row[tid] = A.part_ptr[it.seq_begin + tid] + it.part_row;
 
     // Q^T operand: sequence row mb*16+i, dims 32*ks + 8*g .. +7
@@ -707,7 +774,9 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
         for (int db = 0; db < 8; db++) {
             const h4 a = lds_read_tr(&sm.v[w][(4 * g + (i >> 2)) * VPITCH + 16 * db + 4 * (i & 3)]);
             oacc[0][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[0], oacc[0][db], 0, 0, 0);
-            if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1], oacc[1][db], 0, 0, 0);
+            if constexpr (MB > 1) {
+                if (two) oacc[1][db] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[1], oacc[1][db], 0, 0, 0);
+            }
         }
         __builtin_amdgcn_wave_barrier();
 
@@ -1105,14 +1174,27 @@ struct DecodeRest {
     float* part;
     const int32_t* part_ptr;
     int32_t* counters;
+    const half_t* k_new;  // fused decode step only
+    const half_t* v_new;
 };
 constexpr int kFlagFuseMerge = 1, kFlagPerWave = 2, kFlagStreamNt = 4;
 
-template <int C>
-__global__ __launch_bounds__(WG, 2) void decode_kernel(const WorkItem* stream_items, const WorkItem* shared_items,
-                                                       const half_t* kpool, const half_t* vpool, const half_t* q,
-                                                       int n_shared_wgs, int H, int delta_tokens, int flags,
-                                                       float scale_log2, int n_stream_items, const DecodeRest rest) {
+// Workgroup b of a launch runs on XCD b % 8 of this part, and every XCD has an L2 of its own.
+// The row tiles of one (shared segment, head) read the same K/V: they should meet in one L2 and
+// run at about the same time.  Shared workgroup b therefore takes unit
+//   u = (b % 8) * ceil-share + b / 8      (XCD x works through a contiguous range of units)
+// of the head-major order u = head * n_items + item, in which the row tiles of a segment (adjacent
+// in the item list) are neighbours -- whatever the number of heads is.
+__device__ __forceinline__ int xcd_unit(int b, int n) {
+    const int x = b & 7, q = n >> 3, r = n & 7;
+    return x * q + (x < r ? x : r) + (b >> 3);
+}
+
+template <int C, int MIX, bool APPEND>
+__global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void decode_kernel(
+    const WorkItem* stream_items, const WorkItem* shared_items, const half_t* kpool, const half_t* vpool,
+    const half_t* q, int n_shared_wgs, int H, int delta_tokens, int flags, float scale_log2,
+    int n_stream_items, const DecodeRest rest) {
     DecodeArgs A;
     A.q = q; A.kpool = kpool; A.vpool = vpool; A.out = rest.out; A.part = rest.part;
     A.shared_items = shared_items; A.stream_items = stream_items; A.slots = rest.slots;
@@ -1122,28 +1204,38 @@ __global__ __launch_bounds__(WG, 2) void decode_kernel(const WorkItem* stream_it
     A.n_stream_items = n_stream_items;
     A.stream_per_wave = (flags & kFlagPerWave) ? 1 : 0;
     A.stream_nt = (flags & kFlagStreamNt) ? 1 : 0;
-    __shared__ DecodeLds lds;
+    A.k_new = rest.k_new; A.v_new = rest.v_new;
+    __shared__ DecodeLds<MIX> lds;
     const int bid = blockIdx.x;
-    if (bid < A.n_shared_wgs) {
-        const WorkItem* gi = A.shared_items + bid / A.H;
-        if (gi->flags & kItemWide) {
-            // up to 64 sequences: 16 rows per wave keep all four waves busy
-            if (gi->n_rows <= 64) {
-                wide_path<C, 1>(A, gi, bid % A.H, lds.wd);
+    if (MIX != kMixStream && bid < A.n_shared_wgs) {
+        if constexpr (MIX != kMixStream) {
+            const int unit = xcd_unit(bid, A.n_shared_wgs);
+            const int n_items = A.n_shared_wgs / A.H;
+            const int h = unit / n_items;
+            const WorkItem* gi = A.shared_items + (unit - h * n_items);
+            if constexpr (MIX == kMixFull) {
+                if (gi->flags & kItemWide) {
+                    // up to 64 sequences: 16 rows per wave keep all four waves busy
+                    if (gi->n_rows <= 64) {
+                        wide_path<C, 1>(A, gi, h, lds.wd);
+                    } else {
+                        wide_path<C, 2>(A, gi, h, lds.wd);
+                    }
+                } else {
+                    shared_path<C, 2>(A, gi, h, lds.sh);
+                }
             } else {
-                wide_path<C, 2>(A, gi, bid % A.H, lds.wd);
+                shared_path<C, 1>(A, gi, h, lds.sh);
             }
-        } else {
-            shared_path<C>(A, gi, bid % A.H, lds.sh);
         }
     } else {
         const int sid = bid - A.n_shared_wgs;
         if (A.stream_per_wave) {
             // four consecutive items per workgroup, one per wave, same head
             const int item = 4 * (sid / A.H) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            if (item < A.n_stream_items) stream_path<C, true>(A, A.stream_items + item, sid % A.H, lds.st);
+            if (item < A.n_stream_items) stream_path<C, true, APPEND>(A, A.stream_items + item, sid % A.H, lds.st);
         } else {
-            stream_path<C, false>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
+            stream_path<C, false, APPEND>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
         }
     }
 }
@@ -1259,27 +1351,63 @@ __global__ __launch_bounds__(WG) void put_rows_kernel(const T* __restrict__ k, c
     vpool[dst] = v[src];
 }
 
+// Whole-chunk copies, all pairs in one launch (the beam-search step's tail copies): workgroup y
+// of the grid's second dimension copies pair y of both pools, 16 bytes per thread and step.
+constexpr int COPY_PAIRS = 64;
+struct CopyPairs {
+    int32_t src[COPY_PAIRS];
+    int32_t dst[COPY_PAIRS];
+};
+__global__ __launch_bounds__(WG) void copy_chunks_kernel(uint4* __restrict__ kpool, uint4* __restrict__ vpool,
+                                                         CopyPairs pairs, int units_per_chunk) {
+    const size_t src = size_t(pairs.src[blockIdx.y]) * units_per_chunk;
+    const size_t dst = size_t(pairs.dst[blockIdx.y]) * units_per_chunk;
+    for (int u = blockIdx.x * WG + threadIdx.x; u < units_per_chunk; u += gridDim.x * WG) {
+        const uint4 kk = kpool[src + u], vv = vpool[src + u];
+        kpool[dst + u] = kk;
+        vpool[dst + u] = vv;
+    }
+}
+
 // Partial rows of the allocation-free forward.  In host code this name is only a handle for
 // hipGetSymbolAddress: the kernels get the resolved device address as an argument.
 static __device__ __align__(256) float scratch[kScratchBytes / sizeof(float)];
+// Where the read probe would store (it practically never does): its own word, so that a probe on
+// another stream cannot touch a partial row.
+static __device__ __align__(16) uint32_t probe_sink[4];
 
 constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;  // contexts may be created from several threads
 float* g_scratch_ptr[kMaxDevices] = {};
+void* g_probe_sink_ptr[kMaxDevices] = {};
 
 }  // namespace
 
 int scratch_setup(int device) {
     if (device < 0 || device >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
-    if (g_scratch_ptr[device]) return 0;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_scratch_ptr[device] && g_probe_sink_ptr[device]) return 0;
     void* ptr = nullptr;
-    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return static_cast<int>(e);
+    void* sink = nullptr;
+    e = hipGetSymbolAddress(&sink, HIP_SYMBOL(probe_sink));
+    if (e != hipSuccess) return static_cast<int>(e);
+    g_probe_sink_ptr[device] = sink;
     g_scratch_ptr[device] = static_cast<float*>(ptr);
     return 0;
 }
 
 float* scratch_ptr(int device) {
-    return (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+    if (device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    return g_scratch_ptr[device];
+}
+
+void* probe_sink_ptr(int device) {
+    if (device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    return g_probe_sink_ptr[device];
 }
 
 // ---- launchers -----------------------------------------------------------------------------
@@ -1310,12 +1438,16 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.n_stream_items = 0;
     d.stream_per_wave = 0;
     d.stream_nt = a.stream_nt ? 1 : 0;
+    d.k_new = static_cast<const half_t*>(a.k_new);
+    d.v_new = static_cast<const half_t*>(a.v_new);
     return d;
 }
 
 int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, bool fuse_merge,
                   hipStream_t st) {
     if (a.stream_per_wave && fuse_merge) return -1;  // waves on their own never meet at a barrier
+    const bool append = a.k_new != nullptr;
+    if (append && (!a.v_new || fuse_merge)) return -1;
     const int stream_groups = a.stream_per_wave ? (n_stream_items + NW - 1) / NW : n_stream_items;
     const int64_t wgs = int64_t(n_shared_items + stream_groups) * a.H;
     if (wgs <= 0) return 0;
@@ -1325,19 +1457,34 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     d.n_stream_items = n_stream_items;
     d.stream_per_wave = a.stream_per_wave ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
-    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters };
+    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters, d.k_new, d.v_new };
     const int flags = (d.fuse_merge ? kFlagFuseMerge : 0) | (d.stream_per_wave ? kFlagPerWave : 0) |
                       (d.stream_nt ? kFlagStreamNt : 0);
-#define CA_DECODE_LAUNCH(CS)                                                                              \
-    hipLaunchKernelGGL(decode_kernel<CS>, grid, block, 0, st, d.stream_items, d.shared_items, d.kpool,   \
-                       d.vpool, d.q, d.n_shared_wgs, d.H, d.delta_tokens, flags, d.scale_log2,           \
+    // the lightest form of the kernel that holds every path this launch takes
+    const int mix = (n_shared_items == 0) ? kMixStream : (a.shared_narrow ? kMixNarrow : kMixFull);
+#define CA_DECODE_LAUNCH(CS, MIX, APP)                                                                    \
+    hipLaunchKernelGGL((decode_kernel<CS, MIX, APP>), grid, block, 0, st, d.stream_items, d.shared_items, \
+                       d.kpool, d.vpool, d.q, d.n_shared_wgs, d.H, d.delta_tokens, flags, d.scale_log2,    \
                        d.n_stream_items, rest)
+#define CA_DECODE_MIX(CS)                                                 \
+    do {                                                                  \
+        if (append) {                                                     \
+            if (mix == kMixStream) CA_DECODE_LAUNCH(CS, kMixStream, true); \
+            else if (mix == kMixNarrow) CA_DECODE_LAUNCH(CS, kMixNarrow, true); \
+            else CA_DECODE_LAUNCH(CS, kMixFull, true);                    \
+        } else {                                                          \
+            if (mix == kMixStream) CA_DECODE_LAUNCH(CS, kMixStream, false); \
+            else if (mix == kMixNarrow) CA_DECODE_LAUNCH(CS, kMixNarrow, false); \
+            else CA_DECODE_LAUNCH(CS, kMixFull, false);                   \
+        }                                                                 \
+    } while (0)
     switch (a.C) {
-        case 32: CA_DECODE_LAUNCH(32); break;
-        case 64: CA_DECODE_LAUNCH(64); break;
-        case 128: CA_DECODE_LAUNCH(128); break;
+        case 32: CA_DECODE_MIX(32); break;
+        case 64: CA_DECODE_MIX(64); break;
+        case 128: CA_DECODE_MIX(128); break;
         default: return -1;
     }
+#undef CA_DECODE_MIX
 #undef CA_DECODE_LAUNCH
     CA_LAUNCH_CHECK();
     return 0;
@@ -1369,9 +1516,9 @@ int launch_upload(void* dst_dev, const void* src_pinned, size_t bytes, hipStream
     return 0;
 }
 
-int launch_read_probe(const void* dev, size_t bytes, int n_cus, void* sink, hipStream_t st) {
+int launch_read_probe(const void* dev, size_t bytes, int n_wgs, void* sink, hipStream_t st) {
     if (bytes < 16 || !sink) return -1;
-    hipLaunchKernelGGL(read_probe_kernel, dim3(n_cus > 0 ? n_cus : 256), dim3(WG), 0, st,
+    hipLaunchKernelGGL(read_probe_kernel, dim3(n_wgs > 0 ? n_wgs : 256), dim3(WG), 0, st,
                        static_cast<const uint4*>(dev), bytes / 16, static_cast<uint32_t*>(sink));
     CA_LAUNCH_CHECK();
     return 0;
@@ -1426,6 +1573,30 @@ int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_toke
                                static_cast<const uint16_t*>(v), static_cast<uint16_t*>(kp),
                                static_cast<uint16_t*>(vp), args, t0, n_copy, a.H, a.C, pieces);
         }
+        CA_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, hipStream_t st) {
+    const size_t chunk_bytes = size_t(a.H) * a.C * a.d * 2;
+    if (chunk_bytes % 16 != 0 || chunk_bytes / 16 > 0x7fffffff) return -1;
+    const int units = static_cast<int>(chunk_bytes / 16);
+    uint4* kp = static_cast<uint4*>(const_cast<void*>(a.kpool));
+    uint4* vp = static_cast<uint4*>(const_cast<void*>(a.vpool));
+    for (int i0 = 0; i0 < n_pairs; i0 += COPY_PAIRS) {
+        const int m = (n_pairs - i0 < COPY_PAIRS) ? (n_pairs - i0) : COPY_PAIRS;
+        CopyPairs pairs;
+        for (int i = 0; i < COPY_PAIRS; i++) {
+            pairs.src[i] = (i < m) ? src_dst[2 * (i0 + i)] : 0;
+            pairs.dst[i] = (i < m) ? src_dst[2 * (i0 + i) + 1] : 0;
+        }
+        // enough workgroups per pair to fill the device with a handful of pairs, two 16-byte
+        // pieces of each pool per thread at least
+        int per_pair = (units + 2 * WG - 1) / (2 * WG);
+        if (per_pair > 128) per_pair = 128;
+        if (per_pair < 1) per_pair = 1;
+        hipLaunchKernelGGL(copy_chunks_kernel, dim3(per_pair, m), dim3(WG), 0, st, kp, vp, pairs, units);
         CA_LAUNCH_CHECK();
     }
     return 0;

@@ -127,6 +127,16 @@ void build_stream_items(Plan& p, int chunk_size, const PlanParams& params) {
     }
     p.n_part_rows = p.part_ptr[n_seqs];
 
+    // the fused decode step lets the stream item that ends a sequence write the new token's row
+    p.tails_streamed = n_seqs > 0;
+    for (int s = 0; s < n_seqs; s++) {
+        if (p.own[s].empty() || p.own[s].back() != p.tail_slot[s]) p.tails_streamed = false;
+    }
+    p.shared_narrow = true;
+    for (const WorkItem& it : p.shared_items) {
+        if ((it.flags & kItemWide) || it.n_rows > 16) p.shared_narrow = false;
+    }
+
     // what the kernels assume about every item
     for (const auto* list : { &p.shared_items, &p.stream_items }) {
         for (const WorkItem& it : *list) {
@@ -148,6 +158,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     p.seq_len.assign(n_seqs, 0);
     p.tail_slot.assign(n_seqs, -1);
     p.tail_fill.assign(n_seqs, 0);
+    p.tail_width.assign(n_seqs, 0);
 
     auto is_shared = [&](const ChunkRow& r) {
         if (params.partition == 2) return false;
@@ -172,6 +183,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 p.seq_len[s] += r.n_tokens;
                 p.tail_slot[s] = r.slot;  // the last row covering s is its tail
                 p.tail_fill[s] = r.n_tokens;
+                p.tail_width[s] = r.seq_end - r.seq_begin;
             }
         }
     }
@@ -229,7 +241,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             // a wide workgroup counts for two: it keeps a compute unit's vector and matrix units
             // busy by itself, and a second one beside it only makes both take twice as long
             const bool wide = run_wide(run);
-            wgs += int64_t(n_segs) * ceil_div(n, wide ? kWideRows : kMaxRows) * std::max(params.n_heads, 1) * (wide ? 2 : 1);
+            const int rows = params.max_item_rows > 0 ? std::min(params.max_item_rows, kMaxRows) : kMaxRows;
+            wgs += int64_t(n_segs) * ceil_div(n, wide ? kWideRows : rows) * std::max(params.n_heads, 1) * (wide ? 2 : 1);
         }
         return wgs;
     };
@@ -310,7 +323,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 n_parts[r0.seq_begin + s]++;
             }
             const bool wide = run_wide(run);
-            const int tile_rows = wide ? kWideRows : kMaxRows;
+            const int tile_rows = wide ? kWideRows : (params.max_item_rows > 0 ? std::min(params.max_item_rows, kMaxRows) : kMaxRows);
             for (int m0 = 0; m0 < n; m0 += tile_rows) {
                 WorkItem it{};
                 it.flags = wide ? kItemWide : 0;
@@ -405,6 +418,9 @@ void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_
             throw std::invalid_argument("tables: the last chunk of a rolled sequence is not full");
         }
         if (p.own[s].empty()) throw std::invalid_argument("tables: sequence without a private last chunk");
+        // a streamed last chunk that covers several sequences (partition 2 or a threshold above 1):
+        // where its successors belong among the rows is the tree's business, not the patch's
+        if (p.tail_width[s] != 1) throw std::invalid_argument("tables: the last chunk of a rolled sequence is not its own");
         rolls[s] = 1;
     }
     for (int s = 0; s < p.n_seqs; s++) {
@@ -423,6 +439,7 @@ void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_
         p.own[s].push_back(new_slots[i]);
         p.tail_slot[s] = new_slots[i];
         p.tail_fill[s] = 0;
+        p.tail_width[s] = 1;
     }
     build_stream_items(p, chunk_size, params);
 }

@@ -79,6 +79,8 @@ struct PlanParams {
     int n_heads = 32;
     int n_cus = 256;
     bool allow_per_wave = true;  // the launch schedule can run stream items one per wave
+    int max_item_rows = 0;       // sequences per (non-wide) shared item, 0 = kMaxRows; 16 keeps every
+                                 // such item within the narrow form of the decode kernel
 };
 
 constexpr int kMaxRows = 32;    // sequences per shared work item (M tile)
@@ -93,6 +95,9 @@ struct Plan {
     int n_part_rows = 0;
     int max_parts_per_seq = 0;
     bool stream_per_wave = false;  // stream items are short and many: one per wave, four per workgroup
+    bool shared_narrow = false;    // no shared item is wide or covers more than 16 sequences
+    bool tails_streamed = false;   // every sequence's last chunk is the last chunk of a stream item
+                                   // (what the fused decode step needs)
     int64_t shared_tokens = 0;   // physical tokens attended chunk-first (per head)
     int64_t stream_tokens = 0;   // tokens attended by stream items (per head, at build time)
     std::vector<WorkItem> shared_items;
@@ -102,6 +107,7 @@ struct Plan {
     std::vector<int32_t> part_ptr;   // [n_seqs + 1]: sequence s owns partial rows part_ptr[s] .. part_ptr[s+1]
     std::vector<int32_t> tail_slot;  // per sequence: slot of its last chunk
     std::vector<int32_t> tail_fill;  // per sequence: tokens in that chunk when built
+    std::vector<int32_t> tail_width; // per sequence: sequences covered by that chunk (host-side only)
 
     // host-side state from which the stream items are (re)generated
     PlanHints hints;
@@ -123,7 +129,8 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
 // sequences' stream items are cut again, partial-row numbering follows; shared items keep their
 // segments.  Only for plans in which no last chunk is attended chunk-first (partition 0 or 2
 // with tpp_threshold >= 1).  Throws std::invalid_argument when that does not hold or an argument
-// does not fit the plan; the plan is unchanged then.
+// does not fit the plan (also: the last chunk of a rolled sequence covers other sequences too, which
+// only rows handed in by hand can produce); the plan is unchanged then.
 void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_tokens,
                 const int32_t* seqs, const int32_t* new_slots, int n);
 

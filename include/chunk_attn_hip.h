@@ -104,7 +104,10 @@ int ca_attention(ca_ctx* ctx, const void* q, void* out, int n_seqs, int partitio
  * that, and with CA_ERR_STATE when the tables are not those of partition 0 in the default
  * schedule (it never rebuilds them).  All contexts on one GPU share the array: calls that
  * overlap on one GPU (different streams or threads) race; calls on one stream are safe.  Nothing
- * in the array needs clearing between calls (every row read is written first). */
+ * in the array needs clearing between calls (every row read is written first).
+ * Under graph capture: delta_tokens and the table addresses are kernel arguments of the captured
+ * launches, so a captured forward replays the sequence lengths it was captured with.  Capture
+ * again after every ca_append_kv / ca_decode_step, ca_ctx_roll_tails or refresh. */
 #define CA_NOALLOC_SCRATCH_BYTES (32u << 20)
 int ca_attention_noalloc(ca_ctx* ctx, const void* q, void* out, int n_seqs, void* stream);
 
@@ -120,6 +123,20 @@ int ca_attn_seqs_first(ca_ctx* ctx, const void* q, void* out, int n_seqs, void* 
 /* Replaces append_kv(ctx, keys, values) (kernel_cuda.cu:1273-1318): writes one new K/V row
  * per sequence at position seq_len + delta_tokens.  Does not change delta_tokens. */
 int ca_append_kv(ca_ctx* ctx, const void* k, const void* v, int n_seqs, void* stream);
+
+/* One decode step of the reference's attention layer in one call: Attention::append_token's
+ * device half (attention.cpp:80-114 -> append_kv, kernel_cuda.cu:1273-1318) followed by
+ * forward (attention.cpp:57-78 -> attention, kernel_cuda.cu:1320-1329), i.e. exactly
+ *   ca_append_kv(k, v); ca_ctx_set_delta_tokens(delta_tokens + 1); ca_attention(q, out, partition 0)
+ * with the same results in `out` and in the pools, bit for bit.  k, v: the new token's rows
+ * [n_seqs, n_heads, d_head]; q attends every token including the new one.  When every sequence's
+ * last chunk is streamed per sequence (always, with trees built by ca_tree_* / the Attention class
+ * and tpp_threshold >= 1) no append launch is made: the workgroup that streams a sequence's last
+ * chunk takes the new row from k / v and writes it into the pool on the way.  Otherwise the two
+ * launches are made here.  Same preconditions as ca_append_kv (a free row in every last chunk:
+ * reserve and refresh / ca_ctx_roll_tails first); delta_tokens is advanced by one on success. */
+int ca_decode_step(ca_ctx* ctx, const void* q, const void* k, const void* v, void* out, int n_seqs,
+                   void* stream);
 
 /* Replaces rotary_embedding(positions, query, key, head_size, cos_sin_cache, is_neox)
  * (cpp/chunk_attn/pos_encoding_kernels.cu:94-139, bound as chunk_attn.ops.rotary_embedding in
@@ -167,6 +184,11 @@ int ca_scatter_kv(ca_ctx* ctx, const void* k, const void* v, int n_tokens, int t
 
 /* Device copy of one chunk's K and V (reference Chunk::deep_copy, chunk.cpp:93-107). */
 int ca_copy_chunk(ca_ctx* ctx, int src_slot, int dst_slot, void* stream);
+/* The same for n_pairs chunks in one launch (per 64 pairs): chunk src_dst[2i] is copied onto chunk
+ * src_dst[2i+1] in both pools (host array; what the loops over deep_copy in reference
+ * Attention::duplicate and append_completion do, attention.cpp:227-261,287-313).  No destination
+ * may be the source or the destination of another pair (CA_ERR_INVALID). */
+int ca_copy_chunks(ca_ctx* ctx, const int32_t* src_dst, int n_pairs, void* stream);
 
 /* K/V rows to explicit places, one launch: row i of k and v ([n_rows, n_heads, d_head] on the
  * device) goes to row slot_row[2i+1] of chunk slot_row[2i] (host array).  The device half of the
@@ -201,12 +223,8 @@ int ca_ctx_set_schedule(ca_ctx* ctx, int mode);
  * ca_ctx_read_timing returns the accumulated milliseconds of the decode launch in *shared_ms
  * and of the merge launch in *merge_ms (*stream_ms stays 0).  mode 2: ca_attention runs as
  * three separately timed launches (chunk-first, sequence-first, merge) and the three
- * accumulators are filled; for phase analysis, slower than the normal forward.  mode 3:
- * ca_attention issues only the decode launch (no merge: sequences with more than one partial
- * get no output) and records nothing, so that a caller can time a back-to-back train of that
- * launch between two events of its own.  mode 4: the same for the sequence-first phase alone:
- * ca_attention issues one launch over the stream items only (sequences whose output needs a
- * merge get none). */
+ * accumulators are filled; for phase analysis, slower than the normal forward.  Every mode
+ * writes the complete output. */
 int ca_ctx_set_timing(ca_ctx* ctx, int mode);
 int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double* merge_ms,
                        int64_t* calls, int reset);
@@ -216,12 +234,6 @@ int ca_ctx_read_timing(ca_ctx* ctx, double* shared_ms, double* stream_ms, double
  * (kernel_cuda.cu:1334-1433).  Process-wide, off by default.  Enabling loads the roctx library
  * at run time; CA_ERR_STATE when none is found. */
 int ca_set_markers(int enable);
-
-/* Measurement aid with no counterpart in the reference: one launch on `stream` that reads
- * `bytes` of device memory at `dev` (16-byte aligned, at least 16 bytes) with plain streaming
- * loads and keeps nothing: the read rate a kernel with no structure reaches on this GPU, for
- * benchmarks to quote beside the published peak. */
-int ca_ctx_read_probe(ca_ctx* ctx, const void* dev, size_t bytes, void* stream);
 
 /* Numbers describing the current tables. */
 typedef struct ca_plan_info {
@@ -257,6 +269,23 @@ int ca_ctx_export_partials(ca_ctx* ctx, float* maxs, float* sums, float* attns, 
 /* Raw copy of the partial-row buffer ([n_part_rows][n_heads][160] floats: max, sum, 2 unused,
  * 128 acc in base-2 units, 28 unused) to the host, for inspection.  Synchronises the stream. */
 int ca_ctx_read_partials_raw(ca_ctx* ctx, float* out, int64_t n_floats, void* stream);
+
+/* ---- measurement aids: for benchmarks, not for callers --------------------------------- */
+
+/* Parts of a forward launched alone so that a benchmark can time a back-to-back train of them
+ * between two events of its own.  The output is NOT complete afterwards (sequences whose output
+ * needs the merge launch get none).  what 0: the decode launch without the merge launch; 1: only
+ * its sequence-first workgroups (the stream items); 2: only its chunk-first workgroups.  Needs
+ * tables of partition 0 in the default schedule; never rebuilds them.  No counterpart in the
+ * reference. */
+int ca_bench_decode_launch(ca_ctx* ctx, const void* q, void* out, int n_seqs, int what, void* stream);
+
+/* One launch on `stream` that reads `bytes` of device memory at `dev` (16-byte aligned, at least 16
+ * bytes) with non-temporal 16-byte loads, wgs_per_cu (1 .. 8) workgroups of 256 threads per compute
+ * unit, eight loads per lane in flight, and keeps nothing: the read rate a kernel with no structure
+ * reaches on this GPU, for benchmarks to quote beside the published peak.  No counterpart in the
+ * reference. */
+int ca_bench_read_probe(ca_ctx* ctx, const void* dev, size_t bytes, int wgs_per_cu, void* stream);
 
 /* ---- host-only table builder (no device needed) ---------------------------------------- */
 

@@ -345,13 +345,14 @@ def test_read_probe_reads_and_checks_its_arguments():
     buf = torch.arange(1 << 18, dtype=torch.int64, device=dev())
     before = buf.clone()
     st = torch.cuda.current_stream().cuda_stream
-    for n_bytes in (16, 4096 + 16, buf.numel() * 8):
-        attn.ctx.read_probe(buf.data_ptr(), n_bytes, st)
+    for n_bytes, per_cu in ((16, 1), (4096 + 16, 2), (buf.numel() * 8, 1), (buf.numel() * 8, 4)):
+        attn.ctx.bench_read_probe(buf.data_ptr(), n_bytes, per_cu, st)
     torch.cuda.synchronize()
     assert torch.equal(buf, before)
-    for ptr, n_bytes in ((buf.data_ptr() + 8, 64), (buf.data_ptr(), 8), (0, 64)):
+    for ptr, n_bytes, per_cu in ((buf.data_ptr() + 8, 64, 1), (buf.data_ptr(), 8, 1), (0, 64, 1),
+                                 (buf.data_ptr(), 64, 0), (buf.data_ptr(), 64, 9)):
         with pytest.raises(capi.ChunkAttnError) as e:
-            attn.ctx.read_probe(ptr, n_bytes, st)
+            attn.ctx.bench_read_probe(ptr, n_bytes, per_cu, st)
         assert e.value.code == -1
 
 
@@ -504,7 +505,8 @@ def test_stream_hint_does_not_change_results():
 
 
 def test_timing_modes_leave_results_alone():
-    # HIP-event timing inside the library (modes 1, 2) and the launch-only measurement aids (3, 4)
+    # HIP-event timing inside the library (modes 1, 2): every mode writes the complete output.  The
+    # launch-only measurement aids are entry points of their own and leave the context as it was.
     w = synth.prefix_workload("timing", 6, 64, 256, 200, n_heads=4)
     attn, _ = load_workload(w)
     q = to_dev(w.q())
@@ -521,11 +523,14 @@ def test_timing_modes_leave_results_alone():
         if mode == 2:
             assert t["stream_ms"] > 0
         assert torch.equal(out, want)
-    for mode in (3, 4):   # partial work only: outputs are not complete, nothing is recorded
-        attn.ctx.set_timing(mode)
-        attn.ctx.attention(q.data_ptr(), out.data_ptr(), w.n_seqs, 0, stream)
-        assert attn.ctx.read_timing(reset=True)["calls"] == 0
     attn.ctx.set_timing(0)
-    assert torch.equal(attn.forward(q), want)
+    scratch_out = torch.empty_like(q)
+    for what in (0, 1, 2):   # partial work only: outputs are not complete, nothing is recorded
+        attn.ctx.bench_decode_launch(q.data_ptr(), scratch_out.data_ptr(), w.n_seqs, what, stream)
+        assert attn.ctx.read_timing(reset=True)["calls"] == 0
     with pytest.raises(capi.ChunkAttnError):
-        attn.ctx.set_timing(5)
+        attn.ctx.bench_decode_launch(q.data_ptr(), scratch_out.data_ptr(), w.n_seqs, 3, stream)
+    assert torch.equal(attn.forward(q), want)
+    for mode in (3, 4, 5):   # ca_attention has no mode that leaves outputs incomplete
+        with pytest.raises(capi.ChunkAttnError):
+            attn.ctx.set_timing(mode)

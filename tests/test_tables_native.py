@@ -341,3 +341,12 @@ def test_roll_tails_rejects_what_it_cannot_patch():
     last_chunks_shared = capi.HostTables(rows, 2, c, 0, 0)   # tpp_threshold 0: every chunk is attended chunk-first
     with pytest.raises(capi.ChunkAttnError):
         last_chunks_shared.roll_tails(2, [0], [9])
+    # a full last chunk that two sequences stream (rows by hand: the tree keeps last chunks private):
+    # where the successors go among the rows is not the patch's to decide
+    shared_tail = np.array([[0, 4, 0, 2]], np.int32)
+    for kw in ({"partition": 2}, {"tpp_threshold": 2}):
+        t2 = capi.HostTables(shared_tail, 2, c, **kw)
+        before2 = t2.plan()
+        with pytest.raises(capi.ChunkAttnError):
+            t2.roll_tails(0, [0, 1], [5, 6])
+        assert_plans_equal(t2.plan(), before2)
