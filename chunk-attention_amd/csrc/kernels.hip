@@ -41,6 +41,18 @@ constexpr int WG = 256;                // threads per workgroup (4 wavefronts of
 constexpr int NW = WG / 64;
 constexpr float NEG_INF = -__builtin_huge_valf();
 
+// Debug builds only (-DCA_TIMELINE): every workgroup of the decode launch leaves four stamps of the
+// device's 100 MHz clock -- start, first K/V data consumed, end -- and its kind, read back through
+// ca_debug_timeline.  Never compiled into the library that ships.
+#ifdef CA_TIMELINE
+__device__ unsigned long long ca_timeline[65536 * 4];
+#define CA_STAMP(slot) do { if (threadIdx.x == 0) ca_timeline[(blockIdx.x & 65535) * 4 + (slot)] = wall_clock64(); } while (0)
+#define CA_STAMP_VALUE(slot, v) do { if (threadIdx.x == 0) ca_timeline[(blockIdx.x & 65535) * 4 + (slot)] = (v); } while (0)
+#else
+#define CA_STAMP(slot) do {} while (0)
+#define CA_STAMP_VALUE(slot, v) do {} while (0)
+#endif
+
 __device__ __forceinline__ float shfl_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -515,6 +527,9 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
             }
             // lane (g, j) now owns the score of row 4*(j % NL) + g
             float s = reduce_rows16<NL>(sc, j) * scale_log2;
+#ifdef CA_TIMELINE
+            if (t == 0 && sub == 0) CA_STAMP(1);
+#endif
             const int row = 4 * (j % NL) + g;
             if (row >= vsub || j >= NL) s = NEG_INF;
             const float m_new = fmaxf(m_run, wave_max(s));
@@ -768,6 +783,9 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
             for (int db = 0; db < 8; db++) oacc[mb][db] *= alpha;
         }
 
+#ifdef CA_TIMELINE
+        if (tb == 0) CA_STAMP(1);
+#endif
         __builtin_amdgcn_wave_barrier();
         // O^T += V^T . P^T : A = V^T (row = dim 16*db + i, k = tokens 4g..4g+3)
 #pragma unroll
@@ -1022,6 +1040,9 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
             stage_full_tile(0);
         }
         __syncthreads();
+#ifdef CA_TIMELINE
+        if (t == 0) CA_STAMP(1);
+#endif
         if (t + 1 < n_tiles) fetch_tile(t + 1);
         if (active) {
             // scores of the 64 tokens for this wave's rows; lane (g, i) gets tokens 16tb + 4g .. +3
@@ -1207,6 +1228,8 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
     A.k_new = rest.k_new; A.v_new = rest.v_new;
     __shared__ DecodeLds<MIX> lds;
     const int bid = blockIdx.x;
+    CA_STAMP(0);
+    CA_STAMP_VALUE(2, (unsigned long long)(bid < A.n_shared_wgs ? 0 : 2));
     if (MIX != kMixStream && bid < A.n_shared_wgs) {
         if constexpr (MIX != kMixStream) {
             const int unit = xcd_unit(bid, A.n_shared_wgs);
@@ -1238,6 +1261,7 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
             stream_path<C, false, APPEND>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
         }
     }
+    CA_STAMP(3);
 }
 
 // one wave per (sequence, head)
@@ -1397,6 +1421,13 @@ int scratch_setup(int device) {
     g_scratch_ptr[device] = static_cast<float*>(ptr);
     return 0;
 }
+
+#ifdef CA_TIMELINE
+extern "C" int ca_debug_timeline(unsigned long long* out, int n_wgs) {
+    if (!out || n_wgs < 0 || n_wgs > 65536) return -1;
+    return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(ca_timeline), size_t(n_wgs) * 4 * sizeof(unsigned long long)));
+}
+#endif
 
 float* scratch_ptr(int device) {
     if (device < 0 || device >= kMaxDevices) return nullptr;

@@ -241,8 +241,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
             // a wide workgroup counts for two: it keeps a compute unit's vector and matrix units
             // busy by itself, and a second one beside it only makes both take twice as long
             const bool wide = run_wide(run);
-            const int rows = params.max_item_rows > 0 ? std::min(params.max_item_rows, kMaxRows) : kMaxRows;
-            wgs += int64_t(n_segs) * ceil_div(n, wide ? kWideRows : rows) * std::max(params.n_heads, 1) * (wide ? 2 : 1);
+            wgs += int64_t(n_segs) * ceil_div(n, wide ? kWideRows : kMaxRows) * std::max(params.n_heads, 1) * (wide ? 2 : 1);
         }
         return wgs;
     };
@@ -323,7 +322,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
                 n_parts[r0.seq_begin + s]++;
             }
             const bool wide = run_wide(run);
-            const int tile_rows = wide ? kWideRows : (params.max_item_rows > 0 ? std::min(params.max_item_rows, kMaxRows) : kMaxRows);
+            const int tile_rows = wide ? kWideRows : kMaxRows;
             for (int m0 = 0; m0 < n; m0 += tile_rows) {
                 WorkItem it{};
                 it.flags = wide ? kItemWide : 0;

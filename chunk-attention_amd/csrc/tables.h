@@ -79,8 +79,6 @@ struct PlanParams {
     int n_heads = 32;
     int n_cus = 256;
     bool allow_per_wave = true;  // the launch schedule can run stream items one per wave
-    int max_item_rows = 0;       // sequences per (non-wide) shared item, 0 = kMaxRows; 16 keeps every
-                                 // such item within the narrow form of the decode kernel
 };
 
 constexpr int kMaxRows = 32;    // sequences per shared work item (M tile)
