@@ -160,6 +160,7 @@ def plain_read_gbps(ctx, n_bytes, torch, reps=20, wgs_per_cu=2):
         res[name] = round(nb / (ms * 1e-3) / 1e9, 1)
         del buf
     del flush
+    res["wgs_per_cu"] = wgs_per_cu
     return res
 
 
@@ -381,11 +382,12 @@ def side_costs(attn, w, torch, capi, operators=False):
     return {**norm, **base}
 
 
-def decode_loop(w, torch, capi, synth, seed, unique_tokens):
+def decode_loop(w, torch, capi, synth, seed, unique_tokens, fused=False):
     """The configuration's decode loop on a fresh cache of the pybind11 class: per step one
     append_token (K/V rows of every sequence into the last chunks; when those are full: reserve,
-    new chunks, tables patched in place) and one forward, host work included.  us_per_step: the
-    loop free-running; per-step figures: a second pass with a device sync after every step."""
+    new chunks, tables patched in place) and one forward, host work included -- or, fused, one
+    decode_step, whose attention launch writes the new rows itself.  us_per_step: the loop
+    free-running; per-step figures: a second pass with a device sync after every step."""
     lw = synth.two_level_workload(w.name + "-loop", 8, 8, w.chunk_size, 1024, 512, unique_tokens,
                                   n_heads=w.n_heads, append_steps=w.append_steps)
     res = {}
@@ -399,8 +401,13 @@ def decode_loop(w, torch, capi, synth, seed, unique_tokens):
         new_chunks, per_step, t0 = [], [], time.perf_counter()
         for t in range(lw.append_steps):
             t1 = time.perf_counter()
-            new_chunks.append(len(attn.append_token(toks[t], kv[t][0], kv[t][1])))
-            attn.forward(q)
+            if fused:
+                before = attn.peak_memory_allocated()
+                attn.decode_step(toks[t], q, kv[t][0], kv[t][1])
+                new_chunks.append(int(attn.peak_memory_allocated() > before))
+            else:
+                new_chunks.append(len(attn.append_token(toks[t], kv[t][0], kv[t][1])))
+                attn.forward(q)
             if timed_per_step:
                 torch.cuda.synchronize()
                 per_step.append((time.perf_counter() - t1) * 1e6)
@@ -413,9 +420,96 @@ def decode_loop(w, torch, capi, synth, seed, unique_tokens):
             res["synced_step_median_us"] = round(plain[len(plain) // 2], 1)
             res["synced_steps_that_added_chunks_us"] = {str(i): round(per_step[i], 1) for i in rolled}
         del attn
-    return {"steps": lw.append_steps, "unique_tokens_at_start": unique_tokens, **res,
-            "chunks_added": int(sum(new_chunks)),
-            "note": "append_token + forward per step through chunk_attn.Attention (pybind11), host work included"}
+    return {"steps": lw.append_steps, "unique_tokens_at_start": unique_tokens, "form": "decode_step" if fused else "append_token + forward",
+            **res, "steps_that_added_chunks": int(sum(1 for x in new_chunks if x)),
+            "note": "per step through chunk_attn.Attention (pybind11), host work included"}
+
+
+def decode_step_us(w, q, torch, capi, seed, steps=48):
+    """One decode step through the C-ABI on a fresh cache, free-running (no sync inside the loop):
+    the two-call form (ca_append_kv, delta_tokens + 1, ca_attention) against the fused one
+    (ca_decode_step).  Few enough steps that no last chunk fills (no table work in the loop)."""
+    res = {}
+    k = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    out = torch.empty_like(q)
+    stream = torch.cuda.current_stream().cuda_stream
+    for fused in (None, False, True):     # None: the forward alone under the same protocol
+        attn = build_cache(w, torch, capi, seed)
+        attn.refresh_kernel_context()
+        ctx, n = attn.ctx, w.n_seqs
+        # free rows in the fullest last chunk (the last row of get_chunks covering a sequence is its tail)
+        fill = {}
+        for slot, n_tok, b, e in attn.get_chunks().tolist():
+            for s in range(b, e):
+                fill[s] = n_tok
+        room = w.chunk_size - max(fill.values())
+        n_steps = max(2, min(steps, room - 1))
+        def one():
+            if fused is None:
+                ctx.attention(q.data_ptr(), out.data_ptr(), n, 0, stream)
+            elif fused:
+                ctx.decode_step(q.data_ptr(), k.data_ptr(), k.data_ptr(), out.data_ptr(), n, stream)
+            else:
+                ctx.append_kv(k.data_ptr(), k.data_ptr(), n, stream)
+                ctx.delta_tokens = ctx.delta_tokens + 1
+                ctx.attention(q.data_ptr(), out.data_ptr(), n, 0, stream)
+        one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_steps - 1):
+            one()
+        torch.cuda.synchronize()
+        res["forward_only_us" if fused is None else ("fused_us" if fused else "two_call_us")] = round((time.perf_counter() - t0) * 1e6 / (n_steps - 1), 2)
+        res["steps"] = n_steps - 1
+        del attn
+    res["note"] = ("append + forward per decode step through the C-ABI, free-running: ca_append_kv + ca_attention (three "
+                   "launches) against ca_decode_step (two: the attention launch writes the new rows)")
+    return res
+
+
+def decode_long(w, torch, capi, seed, steps=2048):
+    """A long decode on the configuration: `steps` tokens appended to every sequence through
+    Attention.decode_step (ctypes class), tables patched at every roll-over, with the re-planning
+    policy off (patch only: work-item sizes stay those of the first step) and on (full rebuild
+    whenever the attended tokens moved by more than 25 % since the last one).  Wall clock per step
+    over the whole run and over its last quarter, host work included."""
+    import numpy as np
+    res = {}
+    per_chunk = w.chunk_size * w.n_heads * w.d_head * 2 * 2
+    need = sum((w.seq_len(s) + steps) // w.chunk_size + 3 for s in range(w.n_seqs)) + 64
+    kz = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    q = torch.from_numpy(w.q(seed)).to("cuda:0")
+    outs = {}
+    for name, percent in (("patch_only", 0), ("replan_25", 25)):
+        attn = capi.Attention(n_heads=w.n_heads, d_head=w.d_head, chunk_size=w.chunk_size,
+                              memory_mb=-(-need * per_chunk // (1 << 20)), dtype=torch.float16, device=torch.device("cuda:0"))
+        for s in range(w.n_seqs):
+            k, v = w.kv(s, seed)
+            attn.add_seq(w.tokens(s), torch.from_numpy(np.ascontiguousarray(k)).to("cuda:0"),
+                         torch.from_numpy(np.ascontiguousarray(v)).to("cuda:0"))
+        attn.ctx.set_replan(percent)
+        attn.forward(q)
+        torch.cuda.synchronize()
+        marks = []
+        t0 = time.perf_counter()
+        for t in range(steps):
+            out = attn.decode_step([1_500_000_000 - t * 4096 - s for s in range(w.n_seqs)], q, kz, kz)
+            if (t + 1) % (steps // 4) == 0:
+                torch.cuda.synchronize()
+                marks.append(time.perf_counter())
+        full, patches = attn.ctx.table_stats()
+        info = attn.ctx.plan_info()
+        res[name] = {"us_per_step": round((marks[-1] - t0) * 1e6 / steps, 2),
+                     "last_quarter_us_per_step": round((marks[-1] - marks[-2]) * 1e6 / (steps // 4), 2),
+                     "full_builds": full, "patches": patches,
+                     "final_work_items": [info.n_shared_items, info.n_stream_items], "final_partial_rows": info.n_part_rows}
+        outs[name] = out.float()
+        del attn
+    res["max_abs_diff_between_the_two"] = float((outs["patch_only"] - outs["replan_25"]).abs().max())
+    res["steps"] = steps
+    res["note"] = ("decode_step per step through the ctypes Attention class, zero K/V rows appended; the two runs attend "
+                   "the same cache with differently cut work lists")
+    return res
 
 
 def cpu_baseline(attn, q_np, budget_s, torch):
@@ -458,6 +552,7 @@ def main() -> int:
                     help="also time the layer operators around the attention call (rms_norm, fused_add_rms_norm and "
                          "rotary_embedding on a prefill-sized batch): outside the metric, off by default")
     ap.add_argument("--no-pybind", action="store_true", help="skip timing the forward through the pybind11 class")
+    ap.add_argument("--no-decode-long", action="store_true", help="skip the 2048-step decode with and without re-planning (default configuration only)")
     ap.add_argument("--markers", action="store_true",
                     help="named roctx ranges around refreshes, patches, attention calls and appends (for rocprofv3 --marker-trace)")
     ap.add_argument("--seg-chunks", type=int, default=0)
@@ -474,7 +569,8 @@ def main() -> int:
 
     import numpy as np
     import torch
-    from chunk_attn import capi, synth
+    import synth
+    from chunk_attn import capi
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X: no HIP device visible and there is no CPU fallback", file=sys.stderr)
         return 3
@@ -573,8 +669,10 @@ def main() -> int:
         result["roofline"]["cold_note"] = ("decode launch after 1 GiB of other memory was read, HIP events recorded inside "
                                            "the library around that launch (they add about 2 us: the fraction is a lower bound)")
         result["roofline"]["plain_read_GBps"] = plain_read_gbps(attn.ctx, decode_bytes, torch)
-        result["roofline"]["plain_read_note"] = ("a kernel that only reads (non-temporal 16-byte loads, one workgroup per compute "
-                                                 "unit) over bytes_per_launch bytes under the same two protocols (repeated; after "
+        result["roofline"]["plain_read_1_wg_per_cu_GBps"] = plain_read_gbps(attn.ctx, decode_bytes, torch, wgs_per_cu=1)
+        result["roofline"]["plain_read_note"] = ("a kernel that only reads (non-temporal 16-byte loads, eight per lane in flight, "
+                                                 "two workgroups of 256 threads per compute unit as the decode launch has, and "
+                                                 "one) over bytes_per_launch bytes under the same two protocols (repeated; after "
                                                  "the 1 GiB read) and over 2 GiB, HIP events around the launch")
     if not args.no_pybind:
         pyb_us, pyb_out, pyb_tables = pybind_forward_us(w, q, args.steps, args.warmup, torch, args.seed)
@@ -585,10 +683,14 @@ def main() -> int:
         result["forward_pybind_max_abs_diff"] = float((pyb_out.float() - out.float()).abs().max())
         del pyb_out
     result["per_step_side_costs"] = side_costs(attn, w, torch, capi, args.operators)
+    result["decode_step"] = decode_step_us(w, q, torch, capi, args.seed)
+    if args.config == 1 and not args.no_decode_long:
+        result["decode_long"] = decode_long(w, torch, capi, args.seed)
     if args.config == 3:
         # the two-level configuration's 32 decode steps: as given (tails never fill) and with
         # 100 private tokens, where every tail fills at step 28 (reserve + table rebuild)
-        result["decode_loop"] = [decode_loop(w, torch, capi, synth, args.seed, u) for u in (128, 100)]
+        result["decode_loop"] = [decode_loop(w, torch, capi, synth, args.seed, u, fused) for u in (128, 100)
+                                 for fused in (False, True)]
 
     if not args.no_paged:
         pw = synth.paged_variant(w)

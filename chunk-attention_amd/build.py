@@ -2,6 +2,7 @@
 
   python build.py            # libchunkattn_hip.so (HIP kernels + C-ABI) and chunk_attn_c (pybind11/libtorch module)
   python build.py --no-pybind
+  python build.py --host-sanitize   # host-only half (tables, prefix tree) under ASan + UBSan, for the CPU tests
 
 Outputs go to chunk_attn/lib/.  hipcc cross-compiles, so this runs without a GPU.
 """
@@ -36,11 +37,28 @@ def _run(cmd):
 def build_hip_lib() -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, f) for f in ("kernels.hip", "rotary.hip", "norm.hip", "c_api.cpp", "tables.cpp", "prefix_tree.cpp")]
+    srcs = [os.path.join(CSRC, f) for f in ("kernels.hip", "rotary.hip", "norm.hip", "c_api.cpp", "c_api_host.cpp", "tables.cpp", "prefix_tree.cpp")]
     cmd = [hipcc] + HIP_FLAGS + ["-shared", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
                                   "-o", HIP_LIB] + srcs
     _run(cmd)
     return HIP_LIB
+
+
+HOST_SAN_LIB = os.path.join(LIBDIR, "libchunkattn_host_san.so")
+
+
+def build_host_sanitized() -> str:
+    """The host-only half of the C-ABI (table builder and prefix-tree manager: c_api_host.cpp,
+    tables.cpp, prefix_tree.cpp -- no HIP header, no device code) compiled by g++ with
+    AddressSanitizer and UndefinedBehaviorSanitizer.  A checking build for the CPU tests
+    (tests/test_host_sanitized.py), never loaded by the product."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = [os.path.join(CSRC, f) for f in ("c_api_host.cpp", "tables.cpp", "prefix_tree.cpp")]
+    cmd = [os.environ.get("CXX", "g++"), "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-fno-omit-frame-pointer",
+           "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-o", HOST_SAN_LIB] + srcs
+    _run(cmd)
+    return HOST_SAN_LIB
 
 
 def pybind_target() -> str:
@@ -74,8 +92,14 @@ def build_pybind() -> str:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-pybind", action="store_true")
+    ap.add_argument("--host-sanitize", action="store_true",
+                    help="only build the host-only half of the C-ABI with ASan + UBSan (for tests/test_host_sanitized.py)")
     args = ap.parse_args()
     t0 = time.time()
+    if args.host_sanitize:
+        build_host_sanitized()
+        print("built in %.1f s" % (time.time() - t0))
+        return 0
     build_hip_lib()
     if not args.no_pybind:
         build_pybind()

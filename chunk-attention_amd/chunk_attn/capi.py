@@ -83,6 +83,8 @@ SIGNATURES = {
     "ca_put_kv_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, c_i32_p,
                                       ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
+    "ca_ctx_set_replan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "ca_ctx_table_stats": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]),
     "ca_ctx_set_schedule": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_ctx_set_stream_hint": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "ca_set_markers": (ctypes.c_int, [ctypes.c_int]),
@@ -104,6 +106,7 @@ SIGNATURES = {
     "ca_tables_build_like": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
                                             ctypes.POINTER(ChunkRow), ctypes.c_int, ctypes.c_int]),
     "ca_tables_roll_tails": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, c_i32_p, c_i32_p, ctypes.c_int]),
+    "ca_tables_stale": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64]),
     "ca_tables_destroy": (None, [ctypes.c_void_p]),
     "ca_tables_info": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(PlanInfo)]),
     "ca_tables_plan_sizes": (ctypes.c_int, [ctypes.c_void_p, c_int_p]),
@@ -144,7 +147,12 @@ def load() -> ctypes.CDLL:
                 f"{_LIB_PATH} is missing: build it with `python chunk-attention_amd/build.py` "
                 "(the decode path has no fallback implementation)")
         lib = ctypes.CDLL(_LIB_PATH)
+        # CHUNK_ATTN_HOST_ONLY=1: the library is a checking build of the host-only half (tables and
+        # prefix tree, e.g. the sanitizer build): device entry points are absent and stay unbound
+        host_only = os.environ.get("CHUNK_ATTN_HOST_ONLY") == "1"
         for name, (res, args) in SIGNATURES.items():
+            if host_only and not hasattr(lib, name):
+                continue
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
@@ -403,6 +411,11 @@ class HostTables:
         b, bp = _i32(slots)
         _check(self._lib.ca_tables_roll_tails(self._h, delta_tokens, ap, bp, len(seqs)))
 
+    def stale(self, percent: int = 25, extra_tokens: int = 0) -> bool:
+        """Would the re-planning policy rebuild these tables (attended tokens drifted by more than
+        `percent` per cent since their last full build)?"""
+        return bool(self._lib.ca_tables_stale(self._h, percent, extra_tokens))
+
     def info(self) -> PlanInfo:
         info = PlanInfo()
         _check(self._lib.ca_tables_info(self._h, ctypes.byref(info)))
@@ -559,6 +572,17 @@ class KernelContext:
     def set_stream_hint(self, mode: int) -> None:
         """Non-temporal loads of private chunks: 0 by working-set size (default), 1 always, 2 never."""
         _check(self._lib.ca_ctx_set_stream_hint(self._h, int(mode)))
+
+    def set_replan(self, percent: int) -> None:
+        """Patched tables are rebuilt once the attended tokens drifted by more than `percent` per cent
+        since the last full build (default 25; 0: never)."""
+        _check(self._lib.ca_ctx_set_replan(self._h, int(percent)))
+
+    def table_stats(self) -> Tuple[int, int]:
+        """(full builds, patches) of the device tables since the context was created."""
+        a, b = ctypes.c_int64(), ctypes.c_int64()
+        _check(self._lib.ca_ctx_table_stats(self._h, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
 
     def set_schedule(self, mode: int) -> None:
         """0: producer launch + merge launch (default); 1: single launch, last finisher merges."""

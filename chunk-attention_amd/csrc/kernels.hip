@@ -489,33 +489,30 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
                         // pool, and put it there
                         const int i_new = (vsub - 1) >> 2;
                         const bool mine = ((vsub - 1) & 3) == g;
+                        // both pieces are requested before either is used: one wait, together with
+                        // the tile's own loads, instead of a round trip each
                         const size_t new_off = (size_t(seq) * H + h) * D;
-                        // K, then V: one row piece at a time keeps the register count down
-                        {
-                            const uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
+                        const uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
+                        const uint4 vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
 #pragma unroll
-                            for (int i = 0; i < NL; i++) {
-                                if (i == i_new && mine) kr[i] = kn;
+                        for (int i = 0; i < NL; i++) {
+                            if (i == i_new && mine) {
+                                kr[i] = kn;
+                                vr[i] = vn;
                             }
-                            uint4* kd = const_cast<uint4*>(kp[0]);
-#pragma unroll
-                            for (int cc = 1; cc < CPT; cc++) {
-                                if (i_new / LPC == cc) kd = const_cast<uint4*>(kp[cc]);
-                            }
-                            if (mine) kd[64 * (i_new % LPC)] = kn;
                         }
-                        {
-                            const uint4 vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
+                        uint4* kd = const_cast<uint4*>(kp[0]);
+                        uint4* vd = const_cast<uint4*>(vp[0]);
 #pragma unroll
-                            for (int i = 0; i < NL; i++) {
-                                if (i == i_new && mine) vr[i] = vn;
+                        for (int cc = 1; cc < CPT; cc++) {
+                            if (i_new / LPC == cc) {
+                                kd = const_cast<uint4*>(kp[cc]);
+                                vd = const_cast<uint4*>(vp[cc]);
                             }
-                            uint4* vd = const_cast<uint4*>(vp[0]);
-#pragma unroll
-                            for (int cc = 1; cc < CPT; cc++) {
-                                if (i_new / LPC == cc) vd = const_cast<uint4*>(vp[cc]);
-                            }
-                            if (mine) vd[64 * (i_new % LPC)] = vn;
+                        }
+                        if (mine) {
+                            kd[64 * (i_new % LPC)] = kn;
+                            vd[64 * (i_new % LPC)] = vn;
                         }
                     }
                 }

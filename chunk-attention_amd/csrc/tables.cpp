@@ -9,6 +9,13 @@ void build_ref_tables(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_si
                       int tpp_threshold, RefTables* out) {
     RefTables& t = *out;
     t = RefTables();
+    // rows come from outside the library: every sequence range is checked before it indexes anything
+    for (int i = 0; i < n_rows; i++) {
+        if (rows[i].seq_begin < 0 || rows[i].seq_end > n_seqs || rows[i].seq_begin >= rows[i].seq_end) {
+            throw std::invalid_argument("tables: chunk row with a bad sequence range");
+        }
+    }
+    if (chunk_size <= 0) throw std::invalid_argument("tables: chunk size must be positive");
     t.n_chunks = n_rows;
     // shared = covers more than tpp_threshold sequences (reference kernel_cuda.cu:1343-1349)
     for (int i = 0; i < n_rows; i++) {
@@ -249,6 +256,7 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
     while (base_tiles < 32 && shared_wgs_with(base_tiles) > int64_t(2) * params.n_cus) base_tiles++;
     if (params.keep) base_tiles = params.keep->base_tiles;
     p.hints.base_tiles = base_tiles;
+    p.hints.built_tokens = params.keep ? params.keep->built_tokens : all_tokens;
     auto seg_chunks_for = [&](bool wide) {
         if (params.shared_seg_chunks > 0) return std::min(params.shared_seg_chunks, kMaxItemChunks);
         const int n_tiles = std::min(base_tiles, wide ? 64 : 32);  // 64-token tiles
@@ -441,6 +449,14 @@ void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_
         p.tail_width[s] = 1;
     }
     build_stream_items(p, chunk_size, params);
+}
+
+bool plan_is_stale(const Plan& plan, int percent, int64_t extra_tokens) {
+    if (percent <= 0 || plan.hints.built_tokens <= 0) return false;
+    const int64_t now = plan.shared_tokens + plan.stream_tokens + extra_tokens;
+    const int64_t then = plan.hints.built_tokens;
+    const int64_t diff = now > then ? now - then : then - now;
+    return diff * 100 > int64_t(percent) * then;
 }
 
 }  // namespace ca

@@ -67,6 +67,8 @@ struct PlanHints {
     int base_tiles = 0;     // length of a shared segment in 64-token tiles before per-run adjustments
     int stream_chunks = 0;  // chunks per stream item
     int taper_chunks = 0;   // chunks per stream item of the last sequences, 0: no taper
+    int64_t built_tokens = 0;  // tokens one forward attended (shared once, private per owner) when
+                               // these sizes were derived: how far a patched plan has drifted from them
 };
 
 struct PlanParams {
@@ -131,5 +133,12 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
 // only rows handed in by hand can produce); the plan is unchanged then.
 void roll_tails(Plan* plan, int chunk_size, const PlanParams& params, int delta_tokens,
                 const int32_t* seqs, const int32_t* new_slots, int n);
+
+// Re-planning policy for long decodes.  A patched plan keeps the work-item sizes that were derived
+// from the step's size at the last full build (PlanHints); they are worth deriving again once the
+// tokens a forward attends differ from what they were then by more than `percent` per cent
+// (`extra_tokens`: tokens appended since the plan was last patched, i.e. delta_tokens * n_seqs).
+// percent <= 0: never.
+bool plan_is_stale(const Plan& plan, int percent, int64_t extra_tokens = 0);
 
 }  // namespace ca

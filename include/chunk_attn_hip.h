@@ -211,6 +211,16 @@ int ca_ctx_set_plan(ca_ctx* ctx, int shared_seg_chunks, int stream_chunks);
  * the reference (its kernels use plain loads, kernel_cuda.cu:885-1086). */
 int ca_ctx_set_stream_hint(ca_ctx* ctx, int mode);
 
+/* Re-planning policy for long decodes.  ca_ctx_roll_tails keeps the work-item sizes (length of a
+ * shared segment, of a stream item) that the last full build derived from the size of the step, so
+ * that patched and rebuilt tables are the same tables; the reference rebuilds everything at every
+ * roll-over instead (kernel_cuda.cu:1331-1445) and its tables never drift.  Once the tokens one
+ * forward attends differ by more than `percent` per cent from what they were at the last full
+ * build, ca_ctx_roll_tails rebuilds from its own rows (sizes derived afresh) instead of patching.
+ * Default 25; 0: never.  ca_ctx_table_stats counts both kinds since the context was created. */
+int ca_ctx_set_replan(ca_ctx* ctx, int percent);
+int ca_ctx_table_stats(const ca_ctx* ctx, int64_t* full_builds, int64_t* patches);
+
 /* How ca_attention is launched.  0 (default): one launch in which chunk-first and sequence-
  * first workgroups run side by side and write partial rows, then a merge launch.  1: a single
  * launch in which the workgroup that finishes the last partial of a (sequence, head) merges
@@ -310,6 +320,9 @@ int ca_tables_build_like(ca_tables** out, const ca_tables* like, const ca_chunk_
 /* host half of ca_ctx_roll_tails on a built table set (the reference-form tables are not patched) */
 int ca_tables_roll_tails(ca_tables* t, int delta_tokens, const int32_t* seq_idx,
                          const int32_t* new_slots, int n);
+/* 1 when the policy of ca_ctx_set_replan would rebuild these tables: the tokens they attend, plus
+ * extra_tokens appended since, differ from those at their (last full) build by more than percent */
+int ca_tables_stale(const ca_tables* t, int percent, int64_t extra_tokens);
 void ca_tables_destroy(ca_tables* t);
 /* sizes: fills the same struct ca_ctx_plan_info fills */
 int ca_tables_info(const ca_tables* t, ca_plan_info* info);

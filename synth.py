@@ -2,7 +2,8 @@
 sharing, and seeded N(0, sigma) Q/K/V drawn from a counter-based generator (so any slice of
 any tensor can be regenerated independently, on any machine).
 
-Used by bench.py and the tests; nothing here touches the GPU.
+Test and benchmark infrastructure (bench.py, tests/, the smoke run), not part of the package;
+nothing here touches the GPU.
 """
 from __future__ import annotations
 

@@ -3,7 +3,8 @@ its state into numpy for the oracle."""
 import numpy as np
 import torch
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from oracle.attention_ref import CpuAttention, textbook_attention
 
 ATOL, RTOL = 2e-3, 1e-2   # fp16 out, fp32 accumulate: tolerance of the decode path

@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 import torch
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from gpu_helpers import (ATOL, RTOL, assert_close, dev, host_state, load_workload, make_attention,
                          oracle_output, to_dev)
 from oracle.attention_ref import textbook_attention, textbook_partials

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from chunk_attn import synth
+import synth
 from gpu_helpers import (assert_chunk_holds, assert_close, load_workload, oracle_output, oracle_tree_rows,
                          textbook_on_original, to_dev)
 
@@ -80,33 +80,53 @@ def test_config3_sharing_sweep(fraction):
         assert_close(outp[s], want[s])
 
 
-def test_config4_decode_steps():
-    # two-level tree, 36-token private tails so that appends cross a chunk boundary
-    w = synth.two_level_workload("cfg4-100", 8, 8, 64, 1024, 512, 100, append_steps=32)
+@pytest.mark.parametrize("unique,fused", [(100, False), (128, False), (128, True)])
+def test_config4_decode_steps(unique, fused):
+    """The two-level tree and its 32 decode steps: as the configuration states it (128 private
+    tokens: last chunks hold 0 tokens at the start and never fill), and with 100 private tokens,
+    where every last chunk fills and rolls over at step 28.  fused: the steps go through
+    decode_step (append and attention in one launch) instead of append_token + forward."""
+    w = synth.two_level_workload("cfg4-%d" % unique, 8, 8, 64, 1024, 512, unique, append_steps=32)
     attn, _ = load_workload(w)
+    np.testing.assert_array_equal(attn.get_chunks(), oracle_tree_rows(w))
     rng = np.random.default_rng(0)
     for step in range(32):
         k, v = w.append_kv(step)
-        attn.append_token(w.append_tokens(step), to_dev(k), to_dev(v))
+        q = (rng.standard_normal((w.n_seqs, w.n_heads, 128))).astype(np.float16)
+        if fused:
+            out = attn.decode_step(w.append_tokens(step), to_dev(q), to_dev(k), to_dev(v))
+        else:
+            attn.append_token(w.append_tokens(step), to_dev(k), to_dev(v))
         if step in (0, 27, 28, 31):
-            q = (rng.standard_normal((w.n_seqs, w.n_heads, 128))).astype(np.float16)
-            assert_close(attn.forward(to_dev(q)), oracle_output(attn, q))
+            if not fused:
+                out = attn.forward(to_dev(q))
+            assert_close(out, oracle_output(attn, q))
+    rows = attn.get_chunks()
+    assert rows[:, 1].sum() == 1024 + 8 * 512 + 64 * (unique + 32)
+
+
+CFG5_SAMPLES = (0, 63, 64, 127, 128, 129, 255)   # both sides of the 128-row boundaries of the wide items
 
 
 def test_config5_large_batch_properties():
-    # 256 sequences: checked on a sample of sequences against float64 textbook attention
+    """256 sequences over a 4096-token prompt (the chunk-first regime: wide items of 128 rows).
+    K/V are drawn on the device; the sampled sequences are checked against float64 attention over
+    host copies of the tensors that were inserted (never a read-back of the GPU's own pool), the
+    tree against the oracle's tree, sampled chunks against the inserted rows."""
     w = synth.baseline_config(4)
-    attn, _ = load_workload(w)
+    attn, order, kept = load_workload(w, keep=CFG5_SAMPLES)
+    assert order == list(range(w.n_seqs))
+    np.testing.assert_array_equal(attn.get_chunks(), oracle_tree_rows(w))
+    assert_chunk_holds(attn, w, 0, 5, kv=kept[0])                      # a shared chunk
+    assert_chunk_holds(attn, w, 255, 4096 // 64 + 2, kv=kept[255])     # a private chunk of the last sequence
+    assert_chunk_holds(attn, w, 128, 4096 // 64, kv=kept[128])
     q = w.q()
     out = attn.forward(to_dev(q))
+    info = attn.ctx.plan_info()
     out2 = attn.forward(to_dev(q), 2)
     np.testing.assert_allclose(out.float().cpu().numpy(), out2.float().cpu().numpy(), atol=2e-3, rtol=1e-2)
-    from gpu_helpers import host_state
-    from oracle.attention_ref import gather_seq_kv
-    rows, kpool, vpool = host_state(attn, as_float=False)
-    for s in (0, 63, 64, 129, 255):
-        k, v = gather_seq_kv(rows.tolist(), s, kpool, vpool)
-        sc = np.einsum("hd,htd->ht", q[s].astype(np.float64), k.astype(np.float64)) / np.sqrt(128)
-        p = np.exp(sc - sc.max(axis=1, keepdims=True))
-        want = np.einsum("ht,htd->hd", p / p.sum(axis=1, keepdims=True), v.astype(np.float64))
+    assert info.n_shared_chunks == 64 and info.shared_tokens == 4096 and info.stream_tokens == 256 * 256
+    for s in CFG5_SAMPLES:
+        want = textbook_on_original(w, q, s, kv=kept[s])
         assert_close(out[s], want)
+        assert_close(out2[s], want)

@@ -15,8 +15,7 @@ from oracle.attention_ref import textbook_attention
 pytestmark = pytest.mark.gpu
 
 
-def build(c, rng):
-    H = 2
+def build(c, rng, H=2):
     attn = make_attention(H, c, 700)
     root = list(range(3 * c))                                         # shared by everyone
     rk, rv = rng.standard_normal((len(root), H, 128)).astype(np.float16), rng.standard_normal((len(root), H, 128)).astype(np.float16)
@@ -66,3 +65,23 @@ def test_plan_shapes(c):
         for partition in (0, 1, 2):
             assert_close(attn.forward(tq, partition), want)
     assert worst < 2e-3
+
+
+@pytest.mark.parametrize("H", [1, 5, 12, 40])
+def test_head_counts_that_are_no_multiple_of_eight(H):
+    """Chunk-first workgroups are mapped to (work item, head) so that the row tiles of one (segment,
+    head) land on one XCD (workgroup b runs on XCD b % 8): the mapping must cover every (item, head)
+    exactly once for any number of heads and items, which shows as every output row being right."""
+    c = 64
+    rng = np.random.default_rng(400 + H)
+    attn, n, _ = build(c, rng, H)
+    q = rng.standard_normal((n, H, 128)).astype(np.float16)
+    rows, kpool, vpool = host_state(attn)
+    want = textbook_attention(q.astype(np.float32), rows.tolist(), kpool, vpool)
+    tq = to_dev(q)
+    for seg in (0, 1, 3):
+        attn.ctx.set_plan(seg, 0)
+        for partition in (0, 1):
+            out = attn.forward(tq, partition)
+            assert attn.ctx.plan_info().n_shared_items > 0
+            assert_close(out, want)

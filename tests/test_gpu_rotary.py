@@ -11,7 +11,8 @@ import numpy as np
 import pytest
 import torch
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from gpu_helpers import ATOL, RTOL, assert_close, dev, host_state, load_workload, make_attention, to_dev
 from oracle.rotary import cos_sin_cache, rotary_embedding
 

@@ -6,7 +6,8 @@ import random
 import numpy as np
 import pytest
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from oracle.prefix_tree import PrefixTree, build_ref_tables
 from kats import ADD_SEQ_STEPS, TABLE_KAT
 
@@ -350,3 +351,47 @@ def test_roll_tails_rejects_what_it_cannot_patch():
         with pytest.raises(capi.ChunkAttnError):
             t2.roll_tails(0, [0, 1], [5, 6])
         assert_plans_equal(t2.plan(), before2)
+
+
+@pytest.mark.parametrize("cfg,steps", [(0, 1024), (1, 2048), (3, 1024)])
+def test_replanning_policy_keeps_patched_tables_near_fresh_ones(cfg, steps):
+    """A long decode, tables patched at every roll-over (ca_tables_roll_tails) and rebuilt whenever
+    the policy says so (ca_tables_stale, threshold 25 %: what ca_ctx_roll_tails does on the device
+    side).  `stale` is exactly "the attended tokens moved by more than 25 % since the last full
+    build", and while it is false the patched plan has within 10 % of the work items of a plan built
+    afresh from the tree (patch-only drifts to 39 % on the 16-sequence configuration)."""
+    w = synth.baseline_config(cfg)
+    c, n = w.chunk_size, w.n_seqs
+    tree = capi.Tree(c, 1 << 16)
+    for s in range(n):
+        tree.add_seq(w.tokens(s))
+    live = capi.HostTables(tree.get_chunks(), n, c, n_heads=w.n_heads)
+    never = capi.HostTables(tree.get_chunks(), n, c, n_heads=w.n_heads)   # patch-only, for comparison
+    built = live.info().shared_tokens + live.info().stream_tokens
+    delta, rebuilds, worst, worst_never = 0, 0, 0.0, 0.0
+    for step in range(steps):
+        seqs, slots = tree.reserve_tails()
+        if seqs:
+            live.roll_tails(delta, seqs, slots)
+            never.roll_tails(delta, seqs, slots)
+            delta = 0
+            now = live.info().shared_tokens + live.info().stream_tokens
+            assert live.stale(25) == (abs(now - built) * 100 > 25 * built)
+            assert not live.stale(0) and not never.stale(0)          # 0 switches the policy off
+            fresh = capi.HostTables(tree.get_chunks(), n, c, n_heads=w.n_heads)
+            n_fresh = fresh.info().n_shared_items + fresh.info().n_stream_items
+            worst_never = max(worst_never, abs(never.info().n_shared_items + never.info().n_stream_items - n_fresh) / n_fresh)
+            if live.stale(25):
+                live, built, rebuilds = fresh, now, rebuilds + 1
+                assert not live.stale(25)
+            else:
+                worst = max(worst, abs(live.info().n_shared_items + live.info().n_stream_items - n_fresh) / n_fresh)
+        else:
+            # tokens appended since the last patch count as well when the caller passes them
+            assert live.stale(25, delta * n) == (abs(live.info().shared_tokens + live.info().stream_tokens + delta * n - built) * 100 > 25 * built)
+        tree.append_token([5_000_000 + step * 64 + s for s in range(n)])
+        delta += 1
+    assert 3 <= rebuilds <= 12
+    assert worst <= 0.10, worst
+    if cfg == 0:
+        assert worst_never > 0.3

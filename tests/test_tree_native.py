@@ -5,7 +5,8 @@ import random
 import numpy as np
 import pytest
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from oracle.prefix_tree import PrefixTree
 from kats import ADD_SEQ_STEPS, APPEND_CASE, REMOVE_CASE
 

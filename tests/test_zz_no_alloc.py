@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 import torch
 
-from chunk_attn import capi, synth
+import synth
+from chunk_attn import capi
 from gpu_helpers import assert_close, load_workload, oracle_output, to_dev
 
 pytestmark = pytest.mark.gpu
@@ -63,3 +64,50 @@ def test_noalloc_rejects_what_it_cannot_run():
     with pytest.raises(capi.ChunkAttnError) as e:
         a_many.ctx.attention_noalloc(qm.data_ptr(), om.data_ptr(), many.n_seqs, stream)
     assert e.value.code == -1 and "scratch" in str(e.value)
+
+
+def test_noalloc_under_graph_capture_replays_the_eager_result():
+    """What the entry point is for: captured into a HIP graph (where an allocation would fail the
+    capture) and replayed several times, with eager forwards of another cache -- which overwrite
+    the shared scratch -- and synchronisations in between; every replay must equal the eager result.
+    A captured forward is bound to the sequence lengths it was captured with: after an append the
+    replay still gives the old result and the caller captures again."""
+    w = synth.two_level_workload("noalloc-graph", 3, 5, 64, 256, 128, 90, n_heads=8)
+    other = synth.prefix_workload("noalloc-graph-other", 7, 64, 320, 33, n_heads=8)
+    attn, _ = load_workload(w)
+    a_other, _ = load_workload(other)
+    q = w.q()
+    qd = to_dev(q)
+    q_other = to_dev(other.q())
+    want = attn.forward(qd).clone()
+    want_other = a_other.forward(q_other).clone()
+    out = torch.full_like(want, float("nan"))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        attn.ctx.attention_noalloc(qd.data_ptr(), out.data_ptr(), w.n_seqs, side.cuda_stream)   # warm-up
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        attn.ctx.attention_noalloc(qd.data_ptr(), out.data_ptr(), w.n_seqs, torch.cuda.current_stream().cuda_stream)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        out.fill_(float("nan"))
+        got_other = torch.empty_like(want_other)
+        a_other.ctx.attention_noalloc(q_other.data_ptr(), got_other.data_ptr(), other.n_seqs, stream)
+        torch.cuda.synchronize()
+        assert torch.equal(got_other, want_other)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    assert_close(out, oracle_output(attn, q))
+    # an append moves delta_tokens: the captured launches still carry the old value
+    k, v = w.append_kv(0)
+    attn.append_token(w.append_tokens(0), to_dev(k), to_dev(v))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    fresh = torch.empty_like(out)
+    attn.ctx.attention_noalloc(qd.data_ptr(), fresh.data_ptr(), w.n_seqs, stream)
+    assert not torch.equal(fresh, want)
+    assert_close(fresh, oracle_output(attn, q))
