@@ -80,6 +80,8 @@ SIGNATURES = {
                                      ctypes.c_int, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunk": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "ca_copy_chunks": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, ctypes.c_void_p]),
+    "ca_copy_chunks_put_rows": (ctypes.c_int, [ctypes.c_void_p, c_i32_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                               ctypes.c_int, c_i32_p, ctypes.c_void_p]),
     "ca_put_kv_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, c_i32_p,
                                       ctypes.c_void_p]),
     "ca_ctx_set_plan": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
@@ -566,6 +568,14 @@ class KernelContext:
         arr, ptr = _i32([x for p in pairs for x in p])
         _check(self._lib.ca_copy_chunks(self._h, ptr, len(pairs), stream))
 
+    def copy_chunks_put_rows(self, pairs: Sequence[Tuple[int, int]], k_ptr: int, v_ptr: int,
+                             targets: Sequence[Tuple[int, int]], stream: int = 0) -> None:
+        """copy_chunks(pairs) then put_kv_rows(targets): one beam-search step's device work, in one
+        launch when the rows can be left out of the copies."""
+        pa, pp = _i32([x for p in pairs for x in p])
+        ta, tp = _i32([x for t in targets for x in t])
+        _check(self._lib.ca_copy_chunks_put_rows(self._h, pp, len(pairs), k_ptr, v_ptr, len(targets), tp, stream))
+
     def set_plan(self, shared_seg_chunks: int = 0, stream_chunks: int = 0) -> None:
         _check(self._lib.ca_ctx_set_plan(self._h, shared_seg_chunks, stream_chunks))
 
@@ -793,8 +803,7 @@ class Attention:
         k = self._check_kv(k, n, "k")
         v = self._check_kv(v, n, "v")
         pairs, targets = self.tree.append_completion(seq_idx, tokens)
-        self.ctx.copy_chunks(pairs, self._stream())
-        self.ctx.put_kv_rows(k.data_ptr(), v.data_ptr(), targets, self._stream())   # same stream: after the copies
+        self.ctx.copy_chunks_put_rows(pairs, k.data_ptr(), v.data_ptr(), targets, self._stream())
         self.ctx.invalidate()
         return seq_idx
 

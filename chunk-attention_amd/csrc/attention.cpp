@@ -259,14 +259,19 @@ int Attention::append_completion(int seq_idx, std::vector<int>& tokens, torch::T
     std::vector<PrefixTree::RowTarget> rows;
     tree_->append_completion(seq_idx, tokens, &pairs, &rows);
     c10::DeviceGuard guard(t_options_.device());
-    copy_chunks(pairs);  // one launch for every candidate's copy of the tail
-    // row i of k/v is the new token of sequence seq_idx + i (same stream: after the copies)
-    std::vector<int32_t> slot_row;
+    // one launch: every candidate's copy of the tail, and row i of k/v as the new token of
+    // sequence seq_idx + i
+    std::vector<int32_t> flat, slot_row;
+    for (const auto& [src, dst] : pairs) {
+        flat.push_back(src);
+        flat.push_back(dst);
+    }
     for (const auto& r : rows) {
         slot_row.push_back(r.slot);
         slot_row.push_back(r.row);
     }
-    check(ca_put_kv_rows(ctx_, k.data_ptr(), v.data_ptr(), n, slot_row.data(), stream()));
+    check(ca_copy_chunks_put_rows(ctx_, flat.data(), static_cast<int>(pairs.size()), k.data_ptr(), v.data_ptr(), n,
+                                  slot_row.data(), stream()));
     ca_ctx_invalidate(ctx_);  // sequence lengths changed under the device tables
     return seq_idx;
 }

@@ -814,10 +814,10 @@ int ca_scatter_kv(ca_ctx* c, const void* k, const void* v, int n_tokens, int tok
                                         static_cast<hipStream_t>(stream)), "scatter launch");
 }
 
-int ca_copy_chunks(ca_ctx* c, const int32_t* src_dst, int n_pairs, void* stream) {
+namespace {
+int check_copy_pairs(const ca_ctx* c, const int32_t* src_dst, int n_pairs) {
     if (!c || n_pairs < 0) return fail(CA_ERR_INVALID, "bad argument");
-    if (n_pairs == 0) return CA_OK;
-    if (!src_dst) return fail(CA_ERR_INVALID, "null pointer");
+    if (n_pairs > 0 && !src_dst) return fail(CA_ERR_INVALID, "null pointer");
     for (int i = 0; i < n_pairs; i++) {
         const int src = src_dst[2 * i], dst = src_dst[2 * i + 1];
         if (src < 0 || dst < 0 || src >= c->max_chunks || dst >= c->max_chunks) {
@@ -832,16 +832,10 @@ int ca_copy_chunks(ca_ctx* c, const int32_t* src_dst, int n_pairs, void* stream)
         }
     }
     if ((size_t(c->H) * c->C * c->d * 2) % 16 != 0) return fail(CA_ERR_INVALID, "chunk size in bytes must be a multiple of 16");
-    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
-    return launch_rc(ca::launch_copy_chunks(a, src_dst, n_pairs, static_cast<hipStream_t>(stream)), "chunk copy launch");
+    return CA_OK;
 }
 
-int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
-    const int32_t pair[2] = { src_slot, dst_slot };
-    return ca_copy_chunks(c, pair, 1, stream);
-}
-
-int ca_put_kv_rows(ca_ctx* c, const void* k, const void* v, int n_rows, const int32_t* slot_row, void* stream) {
+int check_row_targets(const ca_ctx* c, const void* k, const void* v, int n_rows, const int32_t* slot_row) {
     if (!c || n_rows < 0) return fail(CA_ERR_INVALID, "bad argument");
     if (n_rows == 0) return CA_OK;
     if (!k || !v || !slot_row) return fail(CA_ERR_INVALID, "null pointer");
@@ -851,6 +845,66 @@ int ca_put_kv_rows(ca_ctx* c, const void* k, const void* v, int n_rows, const in
             return fail(CA_ERR_INVALID, "target " + std::to_string(i) + " is outside the pool or the chunk");
         }
     }
+    return CA_OK;
+}
+}  // namespace
+
+int ca_copy_chunks(ca_ctx* c, const int32_t* src_dst, int n_pairs, void* stream) {
+    if (int rc = check_copy_pairs(c, src_dst, n_pairs)) return rc;
+    if (n_pairs == 0) return CA_OK;
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    return launch_rc(ca::launch_copy_chunks(a, src_dst, n_pairs, nullptr, nullptr, nullptr, 0,
+                                            static_cast<hipStream_t>(stream)), "chunk copy launch");
+}
+
+int ca_copy_chunks_put_rows(ca_ctx* c, const int32_t* src_dst, int n_pairs, const void* k, const void* v, int n_rows,
+                            const int32_t* slot_row, void* stream) {
+    if (int rc = check_copy_pairs(c, src_dst, n_pairs)) return rc;
+    if (int rc = check_row_targets(c, k, v, n_rows, slot_row)) return rc;
+    if (n_pairs == 0 && n_rows == 0) return CA_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    // One launch does both when the rows can simply be left out of the copies: the rows fit one
+    // launch's argument block, a written row of a source chunk is written in its destination
+    // chunk as well (else the copy would have to carry the row's old contents over while another
+    // workgroup overwrites them), no chunk gets more than two rows, and no row is written twice.
+    bool one_launch = n_rows <= 64 && n_pairs <= 64 && c->d % 8 == 0;
+    for (int p = 0; one_launch && p < n_pairs; p++) {
+        int rows_seen[2] = { -1, -1 };
+        for (int r = 0; one_launch && r < n_rows; r++) {
+            const int slot = slot_row[2 * r], row = slot_row[2 * r + 1];
+            if (slot != src_dst[2 * p] && slot != src_dst[2 * p + 1]) continue;
+            if (slot == src_dst[2 * p]) {
+                bool also_in_dst = false;
+                for (int q = 0; q < n_rows; q++) also_in_dst |= slot_row[2 * q] == src_dst[2 * p + 1] && slot_row[2 * q + 1] == row;
+                one_launch &= also_in_dst;
+            }
+            if (rows_seen[0] < 0 || rows_seen[0] == row) rows_seen[0] = row;
+            else if (rows_seen[1] < 0 || rows_seen[1] == row) rows_seen[1] = row;
+            else one_launch = false;
+        }
+    }
+    for (int r = 0; one_launch && r < n_rows; r++) {
+        for (int q = 0; q < r; q++) one_launch &= !(slot_row[2 * q] == slot_row[2 * r] && slot_row[2 * q + 1] == slot_row[2 * r + 1]);
+    }
+    if (one_launch) {
+        return launch_rc(ca::launch_copy_chunks(a, src_dst, n_pairs, k, v, slot_row, n_rows, st), "chunk copy and row write launch");
+    }
+    if (n_pairs > 0) {
+        if (int rc = launch_rc(ca::launch_copy_chunks(a, src_dst, n_pairs, nullptr, nullptr, nullptr, 0, st), "chunk copy launch")) return rc;
+    }
+    if (n_rows == 0) return CA_OK;
+    return launch_rc(ca::launch_put_rows(a, k, v, slot_row, n_rows, st), "row write launch");
+}
+
+int ca_copy_chunk(ca_ctx* c, int src_slot, int dst_slot, void* stream) {
+    const int32_t pair[2] = { src_slot, dst_slot };
+    return ca_copy_chunks(c, pair, 1, stream);
+}
+
+int ca_put_kv_rows(ca_ctx* c, const void* k, const void* v, int n_rows, const int32_t* slot_row, void* stream) {
+    if (int rc = check_row_targets(c, k, v, n_rows, slot_row)) return rc;
+    if (n_rows == 0) return CA_OK;
     const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
     return launch_rc(ca::launch_put_rows(a, k, v, slot_row, n_rows, static_cast<hipStream_t>(stream)), "row write launch");
 }

@@ -75,8 +75,12 @@ int launch_append(const LaunchArgs& a, const void* k, const void* v, const int32
 int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_tokens, int tok_begin,
                    const int32_t* slots, int n_slots, hipStream_t st);
 // chunk src_dst[2i] of both pools copied onto chunk src_dst[2i+1], i < n_pairs (host array), one
-// launch per 64 pairs; the pairs must not overlap
-int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, hipStream_t st);
+// launch per 64 pairs; the pairs must not overlap.  With n_rows > 0 (at most 64) the same launch
+// also does what launch_put_rows does for rows i < n_rows of k / v; the token rows it writes are
+// left out of the copies (at most two different rows per pair), so the caller makes sure that a
+// written row of a source chunk is written in the destination chunk too.
+int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, const void* k, const void* v,
+                       const int32_t* slot_row, int n_rows, hipStream_t st);
 // rows i < n of k/v ([n, H, d]) to row slot_row[2i+1] of chunk slot_row[2i] (host array)
 int launch_put_rows(const LaunchArgs& a, const void* k, const void* v, const int32_t* slot_row, int n,
                     hipStream_t st);

@@ -1372,18 +1372,36 @@ __global__ __launch_bounds__(WG) void put_rows_kernel(const T* __restrict__ k, c
     vpool[dst] = v[src];
 }
 
-// Whole-chunk copies, all pairs in one launch (the beam-search step's tail copies): workgroup y
-// of the grid's second dimension copies pair y of both pools, 16 bytes per thread and step.
+// Whole-chunk copies, all pairs in one launch (the beam-search step's tail copies): workgroups
+// (x, y) with y < n_pairs copy pair y of both pools, 16 bytes per thread and step.  Token rows
+// pairs.skip[y][0..1] (-1: none) are left out, in source and destination alike: the same launch
+// writes them.  Workgroups with y >= n_pairs are the row writers: row i of k and v goes to row
+// put.row[i] of chunk put.slot[i] (what put_rows_kernel does).
 constexpr int COPY_PAIRS = 64;
 struct CopyPairs {
     int32_t src[COPY_PAIRS];
     int32_t dst[COPY_PAIRS];
+    int32_t skip[COPY_PAIRS][2];
 };
 __global__ __launch_bounds__(WG) void copy_chunks_kernel(uint4* __restrict__ kpool, uint4* __restrict__ vpool,
-                                                         CopyPairs pairs, int units_per_chunk) {
+                                                         CopyPairs pairs, int n_pairs, int units_per_chunk,
+                                                         int units_per_row, int C, const uint4* __restrict__ k,
+                                                         const uint4* __restrict__ v, PutTargets put, int n_put, int H) {
+    if (int(blockIdx.y) >= n_pairs) {
+        const int idx = (blockIdx.y - n_pairs) * gridDim.x * WG + blockIdx.x * WG + threadIdx.x;
+        if (idx >= n_put * H * units_per_row) return;
+        const int piece = idx % units_per_row, ih = idx / units_per_row, h = ih % H, i = ih / H;
+        const size_t dst = ((size_t(put.slot[i]) * H + h) * C + put.row[i]) * units_per_row + piece;
+        kpool[dst] = k[idx];
+        vpool[dst] = v[idx];
+        return;
+    }
     const size_t src = size_t(pairs.src[blockIdx.y]) * units_per_chunk;
     const size_t dst = size_t(pairs.dst[blockIdx.y]) * units_per_chunk;
+    const int skip0 = pairs.skip[blockIdx.y][0], skip1 = pairs.skip[blockIdx.y][1];
     for (int u = blockIdx.x * WG + threadIdx.x; u < units_per_chunk; u += gridDim.x * WG) {
+        const int row = (u / units_per_row) % C;
+        if (row == skip0 || row == skip1) continue;
         const uint4 kk = kpool[src + u], vv = vpool[src + u];
         kpool[dst + u] = kk;
         vpool[dst + u] = vv;
@@ -1606,25 +1624,49 @@ int launch_scatter(const LaunchArgs& a, const void* k, const void* v, int n_toke
     return 0;
 }
 
-int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, hipStream_t st) {
+int launch_copy_chunks(const LaunchArgs& a, const int32_t* src_dst, int n_pairs, const void* k, const void* v,
+                       const int32_t* slot_row, int n_rows, hipStream_t st) {
     const size_t chunk_bytes = size_t(a.H) * a.C * a.d * 2;
-    if (chunk_bytes % 16 != 0 || chunk_bytes / 16 > 0x7fffffff) return -1;
-    const int units = static_cast<int>(chunk_bytes / 16);
+    if (chunk_bytes % 16 != 0 || chunk_bytes / 16 > 0x7fffffff || (a.d * 2) % 16 != 0) return -1;
+    if (n_rows > PUT_ROWS || (n_rows > 0 && (!k || !v || !slot_row))) return -1;
+    const int units = static_cast<int>(chunk_bytes / 16), units_per_row = a.d * 2 / 16;
     uint4* kp = static_cast<uint4*>(const_cast<void*>(a.kpool));
     uint4* vp = static_cast<uint4*>(const_cast<void*>(a.vpool));
-    for (int i0 = 0; i0 < n_pairs; i0 += COPY_PAIRS) {
+    PutTargets put;
+    for (int i = 0; i < PUT_ROWS; i++) {
+        put.slot[i] = (i < n_rows) ? slot_row[2 * i] : 0;
+        put.row[i] = (i < n_rows) ? slot_row[2 * i + 1] : 0;
+    }
+    // enough workgroups per pair to fill the device with a handful of pairs, two 16-byte
+    // pieces of each pool per thread at least
+    int per_pair = (units + 2 * WG - 1) / (2 * WG);
+    if (per_pair > 128) per_pair = 128;
+    if (per_pair < 1) per_pair = 1;
+    for (int i0 = 0; i0 < n_pairs || (i0 == 0 && n_rows > 0); i0 += COPY_PAIRS) {
         const int m = (n_pairs - i0 < COPY_PAIRS) ? (n_pairs - i0) : COPY_PAIRS;
         CopyPairs pairs;
         for (int i = 0; i < COPY_PAIRS; i++) {
             pairs.src[i] = (i < m) ? src_dst[2 * (i0 + i)] : 0;
             pairs.dst[i] = (i < m) ? src_dst[2 * (i0 + i) + 1] : 0;
+            pairs.skip[i][0] = pairs.skip[i][1] = -1;
+            // rows of this pair's chunks that the row writers own
+            for (int r = 0; i < m && r < n_rows; r++) {
+                if (put.slot[r] != pairs.src[i] && put.slot[r] != pairs.dst[i]) continue;
+                if (pairs.skip[i][0] < 0 || pairs.skip[i][0] == put.row[r]) {
+                    pairs.skip[i][0] = put.row[r];
+                } else if (pairs.skip[i][1] < 0 || pairs.skip[i][1] == put.row[r]) {
+                    pairs.skip[i][1] = put.row[r];
+                } else {
+                    return -1;  // more than two written rows in one pair's chunks: not a beam step
+                }
+            }
         }
-        // enough workgroups per pair to fill the device with a handful of pairs, two 16-byte
-        // pieces of each pool per thread at least
-        int per_pair = (units + 2 * WG - 1) / (2 * WG);
-        if (per_pair > 128) per_pair = 128;
-        if (per_pair < 1) per_pair = 1;
-        hipLaunchKernelGGL(copy_chunks_kernel, dim3(per_pair, m), dim3(WG), 0, st, kp, vp, pairs, units);
+        // the row writers ride along with the first launch
+        const int put_here = (i0 == 0) ? n_rows : 0;
+        const int put_wgs = (put_here * a.H * units_per_row + per_pair * WG - 1) / (per_pair * WG);
+        hipLaunchKernelGGL(copy_chunks_kernel, dim3(per_pair, m + put_wgs), dim3(WG), 0, st, kp, vp, pairs, m, units,
+                           units_per_row, a.C, static_cast<const uint4*>(k), static_cast<const uint4*>(v), put,
+                           put_here, a.H);
         CA_LAUNCH_CHECK();
     }
     return 0;

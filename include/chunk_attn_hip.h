@@ -197,6 +197,14 @@ int ca_copy_chunks(ca_ctx* ctx, const int32_t* src_dst, int n_pairs, void* strea
 int ca_put_kv_rows(ca_ctx* ctx, const void* k, const void* v, int n_rows, const int32_t* slot_row,
                    void* stream);
 
+/* ca_copy_chunks followed by ca_put_kv_rows -- the whole device half of one beam-search step
+ * (reference Attention::append_completion, attention.cpp:227-261: deep copies of the last chunk,
+ * then one row per candidate) -- with the result of making the copies first and the row writes
+ * second.  One launch when the written rows can be left out of the copies (always in a beam
+ * step: every candidate's row has the same index in its own copy of the chunk), two otherwise. */
+int ca_copy_chunks_put_rows(ca_ctx* ctx, const int32_t* src_dst, int n_pairs, const void* k,
+                            const void* v, int n_rows, const int32_t* slot_row, void* stream);
+
 /* Work-list shaping.  0 = choose from the device's compute-unit count and the step's size.
  * shared_seg_chunks = 1 gives one partial row set per shared chunk, the granularity of the
  * reference's partial buffers.  A work item never holds more than 64 chunks: larger values are

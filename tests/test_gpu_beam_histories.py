@@ -84,3 +84,55 @@ def run_history(seed, c, n_ops=50):
 @pytest.mark.parametrize("seed,c", [(0, 32), (1, 64), (2, 128), (3, 32)])
 def test_beam_history(seed, c):
     run_history(seed, c)
+
+
+def test_chunk_copies_and_row_writes_in_one_launch():
+    """ca_copy_chunks / ca_copy_chunks_put_rows against the same steps done one after the other
+    with tensor assignments (reference Chunk::deep_copy, chunk.cpp:93-107, and the row appends of
+    Attention::append_completion, attention.cpp:243,253): the beam-search shape (every candidate's
+    row at the same index of its own copy: one launch), shapes that take two launches (a row
+    written in a source chunk only), and what is rejected."""
+    import torch
+    c, n_slots = 32, 12
+    attn = make_attention(H, c, n_slots)
+    rng = torch.Generator(device="cuda").manual_seed(11)
+    kp, vp = attn.pool_views()
+    st = torch.cuda.current_stream().cuda_stream
+    k = torch.randn((4, H, 128), device="cuda", generator=rng).half()
+    v = torch.randn((4, H, 128), device="cuda", generator=rng).half()
+    cases = [
+        ([(0, 5), (0, 6), (0, 7)], [(0, 9), (5, 9), (6, 9), (7, 9)]),    # a beam step with four candidates
+        ([(1, 8)], [(1, 31), (8, 31), (8, 0)]),                          # two written rows in one destination
+        ([(2, 9), (3, 10)], [(2, 4), (10, 4)]),                          # row of a source only: copies first, then rows
+        ([(2, 9)], [(9, 1), (9, 2), (9, 3)]),                            # three rows in one chunk: two launches
+        ([(4, 11)], []),
+        ([], [(4, 0), (11, 31)]),
+    ]
+    for pairs, targets in cases:
+        kp.copy_(torch.randn(kp.shape, device="cuda", generator=rng).half())
+        vp.copy_(torch.randn(vp.shape, device="cuda", generator=rng).half())
+        want_k, want_v = kp.clone(), vp.clone()
+        for src, dst in pairs:
+            want_k[dst] = want_k[src]
+            want_v[dst] = want_v[src]
+        for i, (slot, row) in enumerate(targets):
+            want_k[slot, :, row] = k[i]
+            want_v[slot, :, row] = v[i]
+        attn.ctx.copy_chunks_put_rows(pairs, k.data_ptr(), v.data_ptr(), targets, st)
+        torch.cuda.synchronize()
+        assert torch.equal(kp, want_k) and torch.equal(vp, want_v), (pairs, targets)
+    # the plain copy entry points
+    before_k, before_v = kp.clone(), vp.clone()
+    attn.ctx.copy_chunks([(0, 3), (1, 4), (2, 5)], st)
+    attn.ctx.copy_chunk(6, 7, st)
+    torch.cuda.synchronize()
+    for src, dst in ((0, 3), (1, 4), (2, 5), (6, 7)):
+        assert torch.equal(kp[dst], before_k[src]) and torch.equal(vp[dst], before_v[src])
+    for untouched in (0, 1, 2, 6, 8, 9, 10, 11):
+        assert torch.equal(kp[untouched], before_k[untouched])
+    for bad in ([(0, 1), (1, 2)], [(0, 2), (1, 2)], [(3, 3)], [(0, attn.max_chunks)]):
+        with pytest.raises(capi.ChunkAttnError) as e:
+            attn.ctx.copy_chunks(bad, st)
+        assert e.value.code == -1
+    with pytest.raises(capi.ChunkAttnError):
+        attn.ctx.copy_chunks_put_rows([(0, 1)], k.data_ptr(), v.data_ptr(), [(0, c)], st)
