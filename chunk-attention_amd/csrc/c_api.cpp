@@ -607,43 +607,84 @@ int ca_attention_noalloc(ca_ctx* c, const void* q, void* out, int n_seqs, void* 
 
 static_assert(CA_NOALLOC_SCRATCH_BYTES == ca::kScratchBytes, "the header's scratch size and the kernels' must agree");
 
-int ca_decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs, void* stream) {
+namespace {
+// The fused decode step: append (optionally with rotary embedding) and attention in one decode
+// launch plus the merge launch.  rope == nullptr: plain append.
+int decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs,
+                const ca::RotaryArgs* rope, hipStream_t st) {
+    if (c->partition != 0 || c->schedule != c->plan_schedule) {
+        if (int rc = build_and_upload(c, 0, st)) return rc;
+    }
+    if (c->schedule == 0 && c->plan.tails_streamed) {
+        // one launch appends and attends: the workgroup that streams a sequence's last chunk
+        // takes the new row from k / v and writes it into the pool on the way
+        c->delta_tokens += 1;
+        ca::LaunchArgs a = launch_args(c, q, out);
+        a.k_new = k;
+        a.v_new = v;
+        a.rope = rope;
+        a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
+        int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
+                                             static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
+        if (rc == CA_OK) rc = run_merge(c, out, st);
+        if (rc != CA_OK) c->delta_tokens -= 1;
+        return rc;
+    }
+    if (rope) {
+        return fail(CA_ERR_STATE, "last chunks are attended chunk-first (or the single-launch schedule is on): "
+                                  "use ca_rope_append_kv, then ca_attention");
+    }
+    // last chunks attended chunk-first, or the single-launch schedule: append, then attend
+    const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
+    if (int rc = launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
+                                             reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
+                                             n_seqs, st), "append launch")) return rc;
+    c->delta_tokens += 1;
+    return run_fused(c, q, out, st);
+}
+
+int check_decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs) {
     if (int rc = check_ready(c, q, n_seqs)) return rc;
     if (int rc = check_attention_shape(c)) return rc;
     if (n_seqs > 0 && (!out || !k || !v)) return fail(CA_ERR_INVALID, "null device pointer");
-    if (n_seqs == 0) return CA_OK;
     for (int s = 0; s < n_seqs; s++) {
         if (c->plan.tail_fill[s] + c->delta_tokens >= c->C) {
             return fail(CA_ERR_STATE, "sequence " + std::to_string(s) + " has no free row in its last chunk: reserve and refresh first");
         }
     }
+    return CA_OK;
+}
+}  // namespace
+
+int ca_decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs, void* stream) {
+    if (int rc = check_decode_step(c, q, k, v, out, n_seqs)) return rc;
+    if (n_seqs == 0) return CA_OK;
     Range range("ca_decode_step");
-    return guarded([&]() -> int {
-        hipStream_t st = static_cast<hipStream_t>(stream);
-        if (c->partition != 0 || c->schedule != c->plan_schedule) {
-            if (int rc = build_and_upload(c, 0, st)) return rc;
+    return guarded([&]() -> int { return decode_step(c, q, k, v, out, n_seqs, nullptr, static_cast<hipStream_t>(stream)); });
+}
+
+int ca_decode_step_rotary(ca_ctx* c, const int64_t* positions, const void* q, const void* k, const void* v,
+                          const void* cos_sin_cache, int max_position, int rot_dim, int is_neox, void* out,
+                          int n_seqs, void* stream) {
+    if (int rc = check_decode_step(c, q, k, v, out, n_seqs)) return rc;
+    if (n_seqs > 0 && !cos_sin_cache) return fail(CA_ERR_INVALID, "null device pointer");
+    if (max_position <= 0 || rot_dim <= 0 || rot_dim > c->d || rot_dim % (is_neox ? 16 : 8) != 0) {
+        return fail(CA_ERR_INVALID, "rot_dim must be a multiple of 16 (NeoX) or 8 (GPT-J) within d_head, max_position positive");
+    }
+    for (int s = 0; s < n_seqs && !positions; s++) {
+        if (c->plan.seq_len[s] + c->delta_tokens >= max_position) {
+            return fail(CA_ERR_INVALID, "sequence " + std::to_string(s) + " is longer than the cos/sin cache");
         }
-        if (c->schedule == 0 && c->plan.tails_streamed) {
-            // one launch appends and attends: the workgroup that streams a sequence's last chunk
-            // takes the new row from k / v and writes it into the pool on the way
-            c->delta_tokens += 1;
-            ca::LaunchArgs a = launch_args(c, q, out);
-            a.k_new = k;
-            a.v_new = v;
-            int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
-                                                 static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
-            if (rc == CA_OK) rc = run_merge(c, out, st);
-            if (rc != CA_OK) c->delta_tokens -= 1;
-            return rc;
-        }
-        // last chunks attended chunk-first, or the single-launch schedule: append, then attend
-        const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
-        if (int rc = launch_rc(ca::launch_append(a, k, v, reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot),
-                                                 reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill),
-                                                 n_seqs, st), "append launch")) return rc;
-        c->delta_tokens += 1;
-        return run_fused(c, q, out, st);
-    });
+    }
+    if (n_seqs == 0) return CA_OK;
+    Range range("ca_decode_step_rotary");
+    ca::RotaryArgs r;
+    r.positions = positions;
+    r.cos_sin_cache = cos_sin_cache;
+    r.rot_dim = rot_dim;
+    r.max_position = max_position;
+    r.is_neox = is_neox != 0;
+    return guarded([&]() -> int { return decode_step(c, q, k, v, out, n_seqs, &r, static_cast<hipStream_t>(stream)); });
 }
 
 int ca_ctx_set_timing(ca_ctx* c, int enable) {

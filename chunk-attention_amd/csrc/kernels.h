@@ -41,6 +41,11 @@ struct LaunchArgs {
     // already counts it).  Needs a work list in which every sequence's last chunk is streamed.
     const void* k_new = nullptr;
     const void* v_new = nullptr;
+    // ... with the rotary embedding of the step's rows folded in: q (as the kernels read it, q
+    // itself stays as it is) and the new K row are rotated for the sequence's position
+    // (rope->positions, or its length before the step).  rope->query / key are not used.
+    const struct RotaryArgs* rope = nullptr;
+    const int32_t* seq_len = nullptr;  // device table: tokens per sequence when the plan was built
 };
 
 // Static device scratch for the entry point that allocates nothing: a file-scope __device__

@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "kernels.h"
+#include "rotary_math.h"
 
 namespace ca {
 namespace {
@@ -220,11 +221,30 @@ struct DecodeArgs {
     int n_stream_items;   // stream items in the list
     int stream_per_wave;  // 1: every wave of a stream workgroup takes an item of its own (needs fuse_merge 0)
     int stream_nt;   // 1: private chunks are read with the non-temporal hint (see LaunchArgs)
-    // Fused decode step (stream_path<.., APPEND>): the newest token of every sequence, [n_seqs, H, D].
+    // Fused decode step (STEP kAppend / kAppendRotary): the newest token of every sequence, [n_seqs, H, D].
     // delta_tokens already counts it; its row in the pool is written by the workgroup that attends it.
     const half_t* k_new;
     const half_t* v_new;
+    // ... with the rotary embedding of the step's rows folded in (STEP 2): q and the new K row are
+    // rotated in registers for the sequence's position (positions[seq], or its length before the
+    // step: seq_len[seq] + delta_tokens - 1); q itself is left as it is in memory
+    const half_t* cos_sin;
+    const int64_t* positions;
+    const int32_t* seq_len;
+    int rot_dim, max_position, neox;
 };
+
+// Decode launches come in three kinds.  kForward: attention over what the pool holds.  kAppend:
+// the fused decode step (see stream_path).  kAppendRotary: the same with rotary embedding.
+constexpr int kForward = 0, kAppend = 1, kAppendRotary = 2;
+
+// The piece own = row[d0 .. d0+7] of a query or new key row of sequence `seq`, rotated.
+__device__ __forceinline__ h8 rotated_piece(const DecodeArgs& A, const half_t* __restrict__ row, int seq, int d0, h8 own) {
+    const int64_t pos = A.positions ? A.positions[seq] : int64_t(A.seq_len[seq]) + A.delta_tokens - 1;
+    const half_t* cs = A.cos_sin + rotary::clamp_pos(pos, A.max_position) * A.rot_dim;
+    return A.neox ? rotary::rotate_piece<true>(row, d0, own, cs, A.rot_dim)
+                  : rotary::rotate_piece<false>(row, d0, own, cs, A.rot_dim);
+}
 
 // Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
 // dims 2l, 2l+1.  Rows are taken NB at a time with all their loads in flight together and
@@ -336,12 +356,12 @@ template <> union __attribute__((aligned(16))) DecodeLds<kMixNarrow> {
 // ---------------------------------------------------------------------------------------
 // PER_WAVE: the wave works alone on its own item (all tiles, no cross-wave combine, no barrier):
 // the form for many short runs, where a workgroup per run would spend its life starting up.
-// APPEND: the fused decode step.  The newest token of the sequence (position len - 1) has no row
+// STEP kAppend / kAppendRotary (APPEND below): the fused decode step.  The newest token of the sequence (position len - 1) has no row
 // in the pool yet: the wave whose tile holds that position takes the row from k_new / v_new
 // instead, and the 16 lanes that hold it store it into the pool.  Nobody else reads that row in
 // this launch (the last chunk of a sequence belongs to exactly one stream item), and the
 // arithmetic is that of a forward over a pool the row was appended to beforehand.
-template <int C, bool PER_WAVE, bool APPEND>
+template <int C, bool PER_WAVE, int STEP>
 __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, StreamPathLds& sm) {
     WorkItem it;  // header only: the inline slots are read from global memory where needed
@@ -372,7 +392,9 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     const int seq = it.seq_begin;
     const int len = it.len0 + A.delta_tokens;
 
-    const h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
+    constexpr bool APPEND = STEP != kForward;
+    h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
+    if constexpr (STEP == kAppendRotary) qv = rotated_piece(A, q + (size_t(seq) * H + h) * D, seq, 8 * j, qv);
 
     float m_run = NEG_INF, l_lane = 0.f;
     float acc[8];
@@ -492,8 +514,11 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
                         // both pieces are requested before either is used: one wait, together with
                         // the tile's own loads, instead of a round trip each
                         const size_t new_off = (size_t(seq) * H + h) * D;
-                        const uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
+                        uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
                         const uint4 vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
+                        if constexpr (STEP == kAppendRotary) {
+                            kn = __builtin_bit_cast(uint4, rotated_piece(A, A.k_new + new_off, seq, 8 * j, __builtin_bit_cast(h8, kn)));
+                        }
 #pragma unroll
                         for (int i = 0; i < NL; i++) {
                             if (i == i_new && mine) {
@@ -661,7 +686,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
 //   of the 16 x 128 V block through the LDS transpose read (lds_read_tr).
 // ---------------------------------------------------------------------------------------
-template <int C, int MBT>
+template <int C, int MBT, bool ROT>
 __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, SharedPathLds<MBT>& sm) {
     constexpr int MB = MBT;  // 16-row blocks of the item
@@ -692,6 +717,9 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
+            if constexpr (ROT) {
+                if (row < it.n_rows) qreg[mb][ks] = rotated_piece(A, qp - 8 * g, it.seq_begin + row, 32 * ks + 8 * g, qreg[mb][ks]);
+            }
         }
     }
 
@@ -916,7 +944,7 @@ __device__ __forceinline__ float max_over_groups(float v) {
     return fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
 }
 
-template <int C, int MBW>
+template <int C, int MBW, bool ROT>
 __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                           int h, WidePathLds& sm) {
     static_assert(MBW == 1 || MBW == 2, "one or two 16-row blocks per wave");
@@ -949,6 +977,9 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
+            if constexpr (ROT) {
+                if (row < it.n_rows) qreg[mb][ks] = rotated_piece(A, qp - 8 * g, it.seq_begin + row, 32 * ks + 8 * g, qreg[mb][ks]);
+            }
         }
     }
     float m_run[MB];
@@ -1194,6 +1225,10 @@ struct DecodeRest {
     int32_t* counters;
     const half_t* k_new;  // fused decode step only
     const half_t* v_new;
+    const half_t* cos_sin;  // ... with rotary embedding only
+    const int64_t* positions;
+    const int32_t* seq_len;
+    int rot_dim, max_position, neox;
 };
 constexpr int kFlagFuseMerge = 1, kFlagPerWave = 2, kFlagStreamNt = 4;
 
@@ -1208,7 +1243,7 @@ __device__ __forceinline__ int xcd_unit(int b, int n) {
     return x * q + (x < r ? x : r) + (b >> 3);
 }
 
-template <int C, int MIX, bool APPEND>
+template <int C, int MIX, int STEP>
 __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void decode_kernel(
     const WorkItem* stream_items, const WorkItem* shared_items, const half_t* kpool, const half_t* vpool,
     const half_t* q, int n_shared_wgs, int H, int delta_tokens, int flags, float scale_log2,
@@ -1223,6 +1258,9 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
     A.stream_per_wave = (flags & kFlagPerWave) ? 1 : 0;
     A.stream_nt = (flags & kFlagStreamNt) ? 1 : 0;
     A.k_new = rest.k_new; A.v_new = rest.v_new;
+    A.cos_sin = rest.cos_sin; A.positions = rest.positions; A.seq_len = rest.seq_len;
+    A.rot_dim = rest.rot_dim; A.max_position = rest.max_position; A.neox = rest.neox;
+    constexpr bool ROT = STEP == kAppendRotary;
     __shared__ DecodeLds<MIX> lds;
     const int bid = blockIdx.x;
     CA_STAMP(0);
@@ -1237,15 +1275,15 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
                 if (gi->flags & kItemWide) {
                     // up to 64 sequences: 16 rows per wave keep all four waves busy
                     if (gi->n_rows <= 64) {
-                        wide_path<C, 1>(A, gi, h, lds.wd);
+                        wide_path<C, 1, ROT>(A, gi, h, lds.wd);
                     } else {
-                        wide_path<C, 2>(A, gi, h, lds.wd);
+                        wide_path<C, 2, ROT>(A, gi, h, lds.wd);
                     }
                 } else {
-                    shared_path<C, 2>(A, gi, h, lds.sh);
+                    shared_path<C, 2, ROT>(A, gi, h, lds.sh);
                 }
             } else {
-                shared_path<C, 1>(A, gi, h, lds.sh);
+                shared_path<C, 1, ROT>(A, gi, h, lds.sh);
             }
         }
     } else {
@@ -1253,9 +1291,9 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
         if (A.stream_per_wave) {
             // four consecutive items per workgroup, one per wave, same head
             const int item = 4 * (sid / A.H) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-            if (item < A.n_stream_items) stream_path<C, true, APPEND>(A, A.stream_items + item, sid % A.H, lds.st);
+            if (item < A.n_stream_items) stream_path<C, true, STEP>(A, A.stream_items + item, sid % A.H, lds.st);
         } else {
-            stream_path<C, false, APPEND>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
+            stream_path<C, false, STEP>(A, A.stream_items + sid / A.H, sid % A.H, lds.st);
         }
     }
     CA_STAMP(3);
@@ -1486,6 +1524,12 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.stream_nt = a.stream_nt ? 1 : 0;
     d.k_new = static_cast<const half_t*>(a.k_new);
     d.v_new = static_cast<const half_t*>(a.v_new);
+    d.cos_sin = a.rope ? static_cast<const half_t*>(a.rope->cos_sin_cache) : nullptr;
+    d.positions = a.rope ? a.rope->positions : nullptr;
+    d.seq_len = a.seq_len;
+    d.rot_dim = a.rope ? a.rope->rot_dim : 0;
+    d.max_position = a.rope ? a.rope->max_position : 0;
+    d.neox = a.rope && a.rope->is_neox ? 1 : 0;
     return d;
 }
 
@@ -1494,6 +1538,14 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     if (a.stream_per_wave && fuse_merge) return -1;  // waves on their own never meet at a barrier
     const bool append = a.k_new != nullptr;
     if (append && (!a.v_new || fuse_merge)) return -1;
+    if (a.rope) {
+        // rotary embedding rides on the fused step only; pieces of 8 halves must pair up
+        if (!append || !a.seq_len || !a.rope->cos_sin_cache || a.rope->max_position <= 0 || a.rope->rot_dim <= 0 ||
+            a.rope->rot_dim > D || a.rope->rot_dim % (a.rope->is_neox ? 16 : 8) != 0) {
+            return -1;
+        }
+    }
+    const int step = !append ? kForward : (a.rope ? kAppendRotary : kAppend);
     const int stream_groups = a.stream_per_wave ? (n_stream_items + NW - 1) / NW : n_stream_items;
     const int64_t wgs = int64_t(n_shared_items + stream_groups) * a.H;
     if (wgs <= 0) return 0;
@@ -1503,26 +1555,27 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     d.n_stream_items = n_stream_items;
     d.stream_per_wave = a.stream_per_wave ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
-    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters, d.k_new, d.v_new };
+    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters, d.k_new, d.v_new, d.cos_sin, d.positions,
+                           d.seq_len, d.rot_dim, d.max_position, d.neox };
     const int flags = (d.fuse_merge ? kFlagFuseMerge : 0) | (d.stream_per_wave ? kFlagPerWave : 0) |
                       (d.stream_nt ? kFlagStreamNt : 0);
     // the lightest form of the kernel that holds every path this launch takes
     const int mix = (n_shared_items == 0) ? kMixStream : (a.shared_narrow ? kMixNarrow : kMixFull);
-#define CA_DECODE_LAUNCH(CS, MIX, APP)                                                                    \
-    hipLaunchKernelGGL((decode_kernel<CS, MIX, APP>), grid, block, 0, st, d.stream_items, d.shared_items, \
-                       d.kpool, d.vpool, d.q, d.n_shared_wgs, d.H, d.delta_tokens, flags, d.scale_log2,    \
+#define CA_DECODE_LAUNCH(CS, MIX, STEP)                                                                    \
+    hipLaunchKernelGGL((decode_kernel<CS, MIX, STEP>), grid, block, 0, st, d.stream_items, d.shared_items, \
+                       d.kpool, d.vpool, d.q, d.n_shared_wgs, d.H, d.delta_tokens, flags, d.scale_log2,     \
                        d.n_stream_items, rest)
+#define CA_DECODE_STEP(CS, MIX)                                           \
+    do {                                                                  \
+        if (step == kForward) CA_DECODE_LAUNCH(CS, MIX, kForward);        \
+        else if (step == kAppend) CA_DECODE_LAUNCH(CS, MIX, kAppend);     \
+        else CA_DECODE_LAUNCH(CS, MIX, kAppendRotary);                    \
+    } while (0)
 #define CA_DECODE_MIX(CS)                                                 \
     do {                                                                  \
-        if (append) {                                                     \
-            if (mix == kMixStream) CA_DECODE_LAUNCH(CS, kMixStream, true); \
-            else if (mix == kMixNarrow) CA_DECODE_LAUNCH(CS, kMixNarrow, true); \
-            else CA_DECODE_LAUNCH(CS, kMixFull, true);                    \
-        } else {                                                          \
-            if (mix == kMixStream) CA_DECODE_LAUNCH(CS, kMixStream, false); \
-            else if (mix == kMixNarrow) CA_DECODE_LAUNCH(CS, kMixNarrow, false); \
-            else CA_DECODE_LAUNCH(CS, kMixFull, false);                   \
-        }                                                                 \
+        if (mix == kMixStream) CA_DECODE_STEP(CS, kMixStream);            \
+        else if (mix == kMixNarrow) CA_DECODE_STEP(CS, kMixNarrow);       \
+        else CA_DECODE_STEP(CS, kMixFull);                                \
     } while (0)
     switch (a.C) {
         case 32: CA_DECODE_MIX(32); break;
@@ -1531,6 +1584,7 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
         default: return -1;
     }
 #undef CA_DECODE_MIX
+#undef CA_DECODE_STEP
 #undef CA_DECODE_LAUNCH
     CA_LAUNCH_CHECK();
     return 0;

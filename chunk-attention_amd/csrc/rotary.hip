@@ -17,30 +17,18 @@
 #include <cstdint>
 
 #include "kernels.h"
+#include "rotary_math.h"
 
 namespace ca {
 namespace {
 
-typedef _Float16 half_t;
-typedef half_t h4 __attribute__((ext_vector_type(4)));
-typedef half_t h8 __attribute__((ext_vector_type(8)));
+using rotary::clamp_pos;
+using rotary::h4;
+using rotary::h8;
+using rotary::half_t;
+using rotary::rot_elem;
 
 constexpr int WG = 256;
-
-__device__ __forceinline__ int64_t clamp_pos(int64_t p, int max_position) {
-    // never read outside the cache, whatever the caller's positions hold
-    return p < 0 ? 0 : (p >= max_position ? int64_t(max_position) - 1 : p);
-}
-
-// Both kernels form the rotation with the same two fp32 operations per element, a rounded
-// product and a fused multiply-add:
-//   x' = fma(x, cos, -(y * sin)),  y' = fma(y, cos, x * sin)
-// (the compiler may still round the result to fp16 in one step or two, so results of the two
-// kernels can differ in the last place)
-__device__ __forceinline__ float rot_elem(float own, float other, float c, float s, bool is_x) {
-    const float t = other * s;
-    return __builtin_fmaf(own, c, is_x ? -t : t);
-}
 
 // One thread rotates one (x, y) pair.  rows: query rows first, then key rows.
 template <bool IS_NEOX>
@@ -147,32 +135,11 @@ __global__ __launch_bounds__(WG) void rope_append_kernel(
     const half_t* in = (role == 0) ? q : k;
     h8 own = *reinterpret_cast<const h8*>(in + src);
     if (8 * piece < rot_dim) {
-        const int embed = rot_dim / 2;
         const int64_t pos = positions ? positions[seq] : int64_t(seq_len[seq]) + delta_tokens;
         const half_t* cs = cache + clamp_pos(pos, max_position) * rot_dim;
-        if constexpr (IS_NEOX) {
-            const bool is_x = 8 * piece < embed;
-            const int r0 = is_x ? 8 * piece : 8 * piece - embed;
-            // the partner piece is read before any lane of this wave stores (one wave holds
-            // whole rows: d/8 lanes per row divide 64), so rotating q in place is safe
-            const h8 other = *reinterpret_cast<const h8*>(in + size_t(sh) * d + (is_x ? r0 + embed : r0));
-            const h8 c8 = *reinterpret_cast<const h8*>(cs + r0);
-            const h8 s8 = *reinterpret_cast<const h8*>(cs + embed + r0);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                own[e] = half_t(rot_elem(float(own[e]), float(other[e]), float(c8[e]), float(s8[e]), is_x));
-            }
-        } else {
-            const h4 c4 = *reinterpret_cast<const h4*>(cs + 4 * piece);
-            const h4 s4 = *reinterpret_cast<const h4*>(cs + embed + 4 * piece);
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float x = float(own[2 * e]), y = float(own[2 * e + 1]);
-                const float c = float(c4[e]), s = float(s4[e]);
-                own[2 * e] = half_t(rot_elem(x, y, c, s, true));
-                own[2 * e + 1] = half_t(rot_elem(y, x, c, s, false));
-            }
-        }
+        // NeoX style: the partner piece is read before any lane of this wave stores (one wave holds
+        // whole rows: d/8 lanes per row divide 64), so rotating q in place is safe
+        own = rotary::rotate_piece<IS_NEOX>(in + size_t(sh) * d, 8 * piece, own, cs, rot_dim);
     }
     if (role == 0) {
         *reinterpret_cast<h8*>(q + src) = own;

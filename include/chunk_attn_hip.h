@@ -138,6 +138,22 @@ int ca_append_kv(ca_ctx* ctx, const void* k, const void* v, int n_seqs, void* st
 int ca_decode_step(ca_ctx* ctx, const void* q, const void* k, const void* v, void* out, int n_seqs,
                    void* stream);
 
+/* ca_decode_step with the rotary embedding of the step's rows folded in: the whole decode branch
+ * of the reference's attention layer (src/chunk_attn/models/llama_hf/modeling_llama.py:62,91-95:
+ * rotary_embedding on the new query/key rows, append_token, forward) in one call and without a
+ * launch of its own for the embedding or the append.  The results in `out` and in the pools are
+ * those of  ca_rope_append_kv(positions, q, k, v, ...); ca_attention(q, out)  (same arithmetic:
+ * fp32 products rounded to fp16 once), but q is only read: the workgroups rotate the rows they
+ * load in registers, and the one that streams a sequence's last chunk rotates the new K row on
+ * its way into the pool.  positions_dev may be NULL (position = the sequence's length before the
+ * step, checked against max_position on the host).  rot_dim: a multiple of 16 (NeoX) or 8
+ * (GPT-J), at most d_head.  CA_ERR_STATE when last chunks are attended chunk-first (tpp_threshold
+ * 0, rows by hand) or the single-launch schedule is on: nothing was done, call ca_rope_append_kv
+ * and ca_attention instead. */
+int ca_decode_step_rotary(ca_ctx* ctx, const int64_t* positions_dev, const void* q, const void* k,
+                          const void* v, const void* cos_sin_cache, int max_position, int rot_dim,
+                          int is_neox, void* out, int n_seqs, void* stream);
+
 /* Replaces rotary_embedding(positions, query, key, head_size, cos_sin_cache, is_neox)
  * (cpp/chunk_attn/pos_encoding_kernels.cu:94-139, bound as chunk_attn.ops.rotary_embedding in
  * cpp/chunk_attn/python_exports_ops.cpp:13): rotates query and key rows in place, fp16 only.
