@@ -428,12 +428,17 @@ def decode_loop(w, torch, capi, synth, seed, unique_tokens, fused=False):
 def decode_step_us(w, q, torch, capi, seed, steps=48):
     """One decode step through the C-ABI on a fresh cache, free-running (no sync inside the loop):
     the two-call form (ca_append_kv, delta_tokens + 1, ca_attention) against the fused one
-    (ca_decode_step).  Few enough steps that no last chunk fills (no table work in the loop)."""
+    (ca_decode_step), the two-call form with the rotary embedding of the step's rows folded into its
+    append (ca_rope_append_kv + ca_attention), and the forward alone under the
+    same protocol beside them (last chunks stay empty there: it attends fewer tokens than the
+    others, whose last chunks fill up step by step).  Few enough steps that no last chunk fills
+    (no table work in the loop)."""
     res = {}
     k = torch.zeros((w.n_seqs, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
     out = torch.empty_like(q)
+    cache = torch.zeros((16384, w.d_head), dtype=torch.float16, device="cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
-    for fused in (None, False, True):     # None: the forward alone under the same protocol
+    for form in ("forward_only", "two_call", "fused", "rotary_two_call"):
         attn = build_cache(w, torch, capi, seed)
         attn.refresh_kernel_context()
         ctx, n = attn.ctx, w.n_seqs
@@ -444,26 +449,35 @@ def decode_step_us(w, q, torch, capi, seed, steps=48):
                 fill[s] = n_tok
         room = w.chunk_size - max(fill.values())
         n_steps = max(2, min(steps, room - 1))
+        qr = q.clone()   # the two-call rotary form rotates it in place
+
         def one():
-            if fused is None:
+            if form == "forward_only":
                 ctx.attention(q.data_ptr(), out.data_ptr(), n, 0, stream)
-            elif fused:
+            elif form == "fused":
                 ctx.decode_step(q.data_ptr(), k.data_ptr(), k.data_ptr(), out.data_ptr(), n, stream)
-            else:
+            elif form == "two_call":
                 ctx.append_kv(k.data_ptr(), k.data_ptr(), n, stream)
                 ctx.delta_tokens = ctx.delta_tokens + 1
                 ctx.attention(q.data_ptr(), out.data_ptr(), n, 0, stream)
+            else:
+                ctx.rope_append_kv(0, qr.data_ptr(), k.data_ptr(), k.data_ptr(), cache.data_ptr(), 16384, w.d_head,
+                                   True, n, stream)
+                ctx.delta_tokens = ctx.delta_tokens + 1
+                ctx.attention(qr.data_ptr(), out.data_ptr(), n, 0, stream)
         one()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(n_steps - 1):
             one()
         torch.cuda.synchronize()
-        res["forward_only_us" if fused is None else ("fused_us" if fused else "two_call_us")] = round((time.perf_counter() - t0) * 1e6 / (n_steps - 1), 2)
+        res[form + "_us"] = round((time.perf_counter() - t0) * 1e6 / (n_steps - 1), 2)
         res["steps"] = n_steps - 1
         del attn
     res["note"] = ("append + forward per decode step through the C-ABI, free-running: ca_append_kv + ca_attention (three "
-                   "launches) against ca_decode_step (two: the attention launch writes the new rows)")
+                   "launches) against ca_decode_step (two: the decode launch attends the new rows from the caller's "
+                   "tensors, the merge launch writes them into the pool); rotary_two_call: ca_rope_append_kv + "
+                   "ca_attention; forward_only attends the cache as built (empty last chunks)")
     return res
 
 

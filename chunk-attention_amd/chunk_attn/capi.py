@@ -65,9 +65,6 @@ SIGNATURES = {
                                     ctypes.c_void_p]),
     "ca_decode_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                       ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]),
-    "ca_decode_step_rotary": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
-                                             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                             ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]),
     "ca_rotary_embedding": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                            ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
@@ -545,18 +542,6 @@ class KernelContext:
         """append_kv + delta_tokens += 1 + attention (partition 0) in one call, one launch fewer."""
         _check(self._lib.ca_decode_step(self._h, q_ptr, k_ptr, v_ptr, out_ptr, n_seqs, stream))
 
-    def decode_step_rotary(self, positions_ptr: int, q_ptr: int, k_ptr: int, v_ptr: int, cache_ptr: int,
-                           max_position: int, rot_dim: int, is_neox: bool, out_ptr: int, n_seqs: int,
-                           stream: int = 0) -> bool:
-        """rope_append_kv + attention in one call without a launch for the embedding or the append
-        (q is only read).  False when the tables do not allow it (nothing was done)."""
-        rc = self._lib.ca_decode_step_rotary(self._h, positions_ptr or None, q_ptr, k_ptr, v_ptr, cache_ptr,
-                                             max_position, rot_dim, int(is_neox), out_ptr, n_seqs, stream)
-        if rc == -3 and "chunk-first" in self._lib.ca_last_error().decode():
-            return False
-        _check(rc)
-        return True
-
     def rope_append_kv(self, positions_ptr: int, q_ptr: int, k_ptr: int, v_ptr: int, cache_ptr: int,
                        max_position: int, rot_dim: int, is_neox: bool, n_seqs: int, stream: int = 0) -> None:
         _check(self._lib.ca_rope_append_kv(self._h, positions_ptr or None, q_ptr, k_ptr, v_ptr, cache_ptr,
@@ -771,40 +756,6 @@ class Attention:
         self.ctx.decode_step(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), n, self._stream())
         self.tree.append_token(tokens)  # reserve inside is a no-op now
         return out
-
-    def decode_step_rotary(self, tokens: Sequence[int], q, k, v, cos_sin_cache, is_neox: bool = True,
-                           positions=None):
-        """append_token_rotary(tokens, q, k, v, ...) followed by forward(q) as one call: the rotary
-        embedding of the new rows and their append ride in the attention launch.  q is left as it
-        is (append_token_rotary rotates it in place).  Returns the output."""
-        import torch
-        n = len(tokens)
-        if self.tree.n_seqs != n:
-            raise RuntimeError("num of seqs is not equal to num of tokens")
-        k = self._check_kv(k, n, "k")
-        v = self._check_kv(v, n, "v")
-        q = self._check_kv(q, n, "q")
-        if cos_sin_cache.dtype != torch.float16 or cos_sin_cache.device != self.device or \
-                cos_sin_cache.dim() != 2 or not cos_sin_cache.is_contiguous():
-            raise RuntimeError("cos_sin_cache must be contiguous fp16 [max_position, rot_dim] on the cache's device")
-        pos_ptr = 0
-        if positions is not None:
-            if positions.dtype != torch.int64 or positions.device != self.device or tuple(positions.shape) != (n,) \
-                    or not positions.is_contiguous():
-                raise RuntimeError(f"positions must be contiguous int64 [{n}] on {self.device}")
-            pos_ptr = positions.data_ptr()
-        self.reserve()
-        self.refresh_kernel_context()
-        out = torch.empty((n, self.n_heads, self.d_head), dtype=q.dtype, device=q.device)
-        if self.ctx.decode_step_rotary(pos_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_sin_cache.data_ptr(),
-                                       cos_sin_cache.shape[0], cos_sin_cache.shape[1], is_neox, out.data_ptr(), n,
-                                       self._stream()):
-            self.tree.append_token(tokens)  # reserve inside is a no-op now
-            return out
-        # last chunks attended chunk-first: the two-call form on a copy of q
-        q = q.clone()
-        self.append_token_rotary(tokens, q, k, v, cos_sin_cache, is_neox, positions)
-        return self.forward(q)
 
     def append_token_rotary(self, tokens: Sequence[int], q, k, v, cos_sin_cache, is_neox: bool = True,
                             positions=None) -> int:

@@ -4,9 +4,8 @@ Mirrors the reference's `LlamaChunkAttention`
 (src/chunk_attn/models/llama_hf/modeling_llama.py:16-113) and its rotary module
 (src/chunk_attn/models/llama_hf/rotary_embedding_vllm.py:43-147) with the same argument
 meaning.  The projections are plain torch matmuls; what differs is the decode branch: the
-rotary embedding of the new query/key rows and the KV append have no launches of their own, they
-ride in the attention launch (`Attention.decode_step_rotary`), where the reference runs a rotary
-launch, an append launch and the attention launches.
+rotary embedding of the new query/key rows and the KV append are one launch
+(`Attention.append_token_rotary`) instead of a rotary launch followed by an append launch.
 Weights are whatever the caller loads; tests use seeded random ones.
 """
 from __future__ import annotations
@@ -84,9 +83,9 @@ class LlamaChunkAttention(nn.Module):
             assert n_tokens == 1
             shape = (batch, self.num_heads, self.head_dim)
             q3, k3, v3 = q.view(shape), k.view(shape), v.view(shape)
-            attn_output = kv_cache.decode_step_rotary([s[-1] for s in seqs], q3.contiguous(), k3, v3,
-                                                      self.rotary_emb.cos_sin_cache, self.rotary_emb.is_neox_style,
-                                                      position_ids.reshape(batch).contiguous()).view(batch, 1, d_hidden)
+            kv_cache.append_token_rotary([s[-1] for s in seqs], q3, k3, v3, self.rotary_emb.cos_sin_cache,
+                                         self.rotary_emb.is_neox_style, position_ids.reshape(batch).contiguous())
+            attn_output = kv_cache.forward(q3).view(batch, 1, d_hidden)
         output = self.o_proj(attn_output)
         kv_cache.reserve()
         kv_cache.refresh_kernel_context(force=False)

@@ -216,46 +216,6 @@ torch::Tensor Attention::decode_step(const std::vector<int>& tokens, torch::Tens
     return output;
 }
 
-torch::Tensor Attention::decode_step_rotary(const std::vector<int>& tokens, torch::Tensor q, torch::Tensor k,
-                                            torch::Tensor v, torch::Tensor cos_sin_cache, bool is_neox,
-                                            c10::optional<torch::Tensor> positions) {
-    if (tree_->tails().size() != tokens.size()) {
-        throw std::runtime_error("num of seqs is not equal to num of tokens");
-    }
-    const int n = static_cast<int>(tokens.size());
-    k = checked_kv(k, n, "k");
-    v = checked_kv(v, n, "v");
-    q = checked_kv(q, n, "q");
-    if (!cos_sin_cache.is_contiguous() || cos_sin_cache.scalar_type() != torch::kFloat16 ||
-        cos_sin_cache.device() != t_options_.device() || cos_sin_cache.dim() != 2) {
-        throw std::runtime_error("cos_sin_cache must be contiguous float16 [max_position, rot_dim] on the cache's device");
-    }
-    const int64_t* pos = nullptr;
-    if (positions.has_value() && positions->defined()) {
-        if (!positions->is_contiguous() || positions->scalar_type() != torch::kInt64 ||
-            positions->device() != t_options_.device() || positions->numel() != n) {
-            throw std::runtime_error("positions must be contiguous int64 [n_seqs] on the cache's device");
-        }
-        pos = positions->data_ptr<int64_t>();
-    }
-    reserve_and_note();
-    refresh_kernel_context();
-    c10::DeviceGuard guard(t_options_.device());
-    torch::Tensor output = torch::empty({ q.size(0), n_heads_, d_head_ }, t_options_);
-    const int rc = ca_decode_step_rotary(ctx_, pos, q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_sin_cache.data_ptr(),
-                                         static_cast<int>(cos_sin_cache.size(0)), static_cast<int>(cos_sin_cache.size(1)),
-                                         is_neox ? 1 : 0, output.data_ptr(), n, stream());
-    if (rc == CA_ERR_STATE && std::string(ca_last_error()).find("chunk-first") != std::string::npos) {
-        // last chunks attended chunk-first: the two-call form, on a copy of q (it rotates in place)
-        torch::Tensor q2 = q.clone();
-        append_token_rotary(tokens, q2, k, v, cos_sin_cache, is_neox, positions);
-        return forward(q2);
-    }
-    check(rc);
-    tree_->append_token_ids(tokens);
-    return output;
-}
-
 torch::Tensor Attention::forward(torch::Tensor q, int partition) {
     if (!q.is_contiguous()) throw std::runtime_error("q is not contiguous");
     if (q.dim() != 3 || q.size(1) != n_heads_ || q.size(2) != d_head_) {

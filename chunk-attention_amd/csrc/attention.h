@@ -50,12 +50,6 @@ class Attention {
     // fewer per step).  q, k, v: [n_seqs, n_heads, d_head].  Returns the output.
     torch::Tensor decode_step(const std::vector<int>& tokens, torch::Tensor q, torch::Tensor k,
                               torch::Tensor v);
-    // decode_step with the rotary embedding of the new rows folded in: append_token_rotary followed
-    // by forward, as one call and without a launch for the embedding or the append.  q is only
-    // read (append_token_rotary rotates it in place).
-    torch::Tensor decode_step_rotary(const std::vector<int>& tokens, torch::Tensor q, torch::Tensor k,
-                                     torch::Tensor v, torch::Tensor cos_sin_cache, bool is_neox = true,
-                                     c10::optional<torch::Tensor> positions = c10::nullopt);
     void refresh_kernel_context(bool force = false);
     std::vector<Chunk*> reserve();
     void clear();

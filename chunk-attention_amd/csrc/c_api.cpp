@@ -384,7 +384,7 @@ int run_stream(ca_ctx* c, const void* q, void* out, hipStream_t st) {
 int run_merge(ca_ctx* c, void* out, hipStream_t st) {
     if (c->plan.n_part_rows == 0) return CA_OK;
     const ca::LaunchArgs a = launch_args(c, nullptr, out);
-    return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
+    return launch_rc(ca::launch_merge(a, c->n_seqs, true, st), "merge launch");
 }
 
 int run_fused(ca_ctx* c, const void* q, void* out, hipStream_t st) {
@@ -602,37 +602,32 @@ int ca_attention_noalloc(ca_ctx* c, const void* q, void* out, int n_seqs, void* 
     if (int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
                                              static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch")) return rc;
     if (c->plan.n_part_rows == 0) return CA_OK;
-    return launch_rc(ca::launch_merge(a, c->n_seqs, st), "merge launch");
+    return launch_rc(ca::launch_merge(a, c->n_seqs, true, st), "merge launch");
 }
 
 static_assert(CA_NOALLOC_SCRATCH_BYTES == ca::kScratchBytes, "the header's scratch size and the kernels' must agree");
 
 namespace {
-// The fused decode step: append (optionally with rotary embedding) and attention in one decode
-// launch plus the merge launch.  rope == nullptr: plain append.
-int decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs,
-                const ca::RotaryArgs* rope, hipStream_t st) {
+// The fused decode step: append and attention in the decode launch plus the merge launch.
+int decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void* out, int n_seqs, hipStream_t st) {
     if (c->partition != 0 || c->schedule != c->plan_schedule) {
         if (int rc = build_and_upload(c, 0, st)) return rc;
     }
     if (c->schedule == 0 && c->plan.tails_streamed) {
-        // one launch appends and attends: the workgroup that streams a sequence's last chunk
-        // takes the new row from k / v and writes it into the pool on the way
+        // no append launch: the workgroup that streams a sequence's last chunk takes the new row
+        // from k / v, and the merge launch writes the rows into the pool
         c->delta_tokens += 1;
         ca::LaunchArgs a = launch_args(c, q, out);
         a.k_new = k;
         a.v_new = v;
-        a.rope = rope;
-        a.seq_len = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_seq_len);
+        a.tail_slot = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_slot);
+        a.tail_fill = reinterpret_cast<const int32_t*>(c->dev_blob + c->off_tail_fill);
         int rc = launch_rc(ca::launch_decode(a, static_cast<int>(c->plan.shared_items.size()),
                                              static_cast<int>(c->plan.stream_items.size()), false, st), "decode launch");
-        if (rc == CA_OK) rc = run_merge(c, out, st);
+        // the merge launch also puts the new rows into the pool (after every read of this step)
+        if (rc == CA_OK) rc = launch_rc(ca::launch_merge(a, c->n_seqs, c->plan.n_part_rows > 0, st), "merge launch");
         if (rc != CA_OK) c->delta_tokens -= 1;
         return rc;
-    }
-    if (rope) {
-        return fail(CA_ERR_STATE, "last chunks are attended chunk-first (or the single-launch schedule is on): "
-                                  "use ca_rope_append_kv, then ca_attention");
     }
     // last chunks attended chunk-first, or the single-launch schedule: append, then attend
     const ca::LaunchArgs a = launch_args(c, nullptr, nullptr);
@@ -660,31 +655,7 @@ int ca_decode_step(ca_ctx* c, const void* q, const void* k, const void* v, void*
     if (int rc = check_decode_step(c, q, k, v, out, n_seqs)) return rc;
     if (n_seqs == 0) return CA_OK;
     Range range("ca_decode_step");
-    return guarded([&]() -> int { return decode_step(c, q, k, v, out, n_seqs, nullptr, static_cast<hipStream_t>(stream)); });
-}
-
-int ca_decode_step_rotary(ca_ctx* c, const int64_t* positions, const void* q, const void* k, const void* v,
-                          const void* cos_sin_cache, int max_position, int rot_dim, int is_neox, void* out,
-                          int n_seqs, void* stream) {
-    if (int rc = check_decode_step(c, q, k, v, out, n_seqs)) return rc;
-    if (n_seqs > 0 && !cos_sin_cache) return fail(CA_ERR_INVALID, "null device pointer");
-    if (max_position <= 0 || rot_dim <= 0 || rot_dim > c->d || rot_dim % (is_neox ? 16 : 8) != 0) {
-        return fail(CA_ERR_INVALID, "rot_dim must be a multiple of 16 (NeoX) or 8 (GPT-J) within d_head, max_position positive");
-    }
-    for (int s = 0; s < n_seqs && !positions; s++) {
-        if (c->plan.seq_len[s] + c->delta_tokens >= max_position) {
-            return fail(CA_ERR_INVALID, "sequence " + std::to_string(s) + " is longer than the cos/sin cache");
-        }
-    }
-    if (n_seqs == 0) return CA_OK;
-    Range range("ca_decode_step_rotary");
-    ca::RotaryArgs r;
-    r.positions = positions;
-    r.cos_sin_cache = cos_sin_cache;
-    r.rot_dim = rot_dim;
-    r.max_position = max_position;
-    r.is_neox = is_neox != 0;
-    return guarded([&]() -> int { return decode_step(c, q, k, v, out, n_seqs, &r, static_cast<hipStream_t>(stream)); });
+    return guarded([&]() -> int { return decode_step(c, q, k, v, out, n_seqs, static_cast<hipStream_t>(stream)); });
 }
 
 int ca_ctx_set_timing(ca_ctx* c, int enable) {

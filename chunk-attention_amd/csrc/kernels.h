@@ -37,15 +37,13 @@ struct LaunchArgs {
     // No shared item of the work list covers more than 16 sequences and none is wide: the launch
     // can take the form of the kernel without the 32-row and wide matrix-core paths.
     bool shared_narrow = false;
-    // Fused decode step: rows [n_seqs, H, 128] of the token appended by this launch (delta_tokens
-    // already counts it).  Needs a work list in which every sequence's last chunk is streamed.
+    // Fused decode step: rows [n_seqs, H, 128] of the token appended by this step (delta_tokens
+    // already counts it).  The decode launch attends them from here, the merge launch writes them
+    // into the pool.  Needs a work list in which every sequence's last chunk is streamed.
     const void* k_new = nullptr;
     const void* v_new = nullptr;
-    // ... with the rotary embedding of the step's rows folded in: q (as the kernels read it, q
-    // itself stays as it is) and the new K row are rotated for the sequence's position
-    // (rope->positions, or its length before the step).  rope->query / key are not used.
-    const struct RotaryArgs* rope = nullptr;
-    const int32_t* seq_len = nullptr;  // device table: tokens per sequence when the plan was built
+    const int32_t* tail_slot = nullptr;  // device tables: slot of every sequence's last chunk and the
+    const int32_t* tail_fill = nullptr;  // tokens it held when the plan was built (fused step's row writes)
 };
 
 // Static device scratch for the entry point that allocates nothing: a file-scope __device__
@@ -65,7 +63,10 @@ void* probe_sink_ptr(int device);
 // its output; otherwise only partial rows (and direct outputs) are written.
 int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, bool fuse_merge,
                   hipStream_t st);
-int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st);
+// The second launch of a forward: merges the partial rows of every (sequence, head) when `merge`,
+// and, for a fused decode step (a.k_new set), writes the step's new K/V rows into the pool
+// (a.tail_slot / a.tail_fill, row tail_fill + delta_tokens - 1).
+int launch_merge(const LaunchArgs& a, int n_seqs, bool merge, hipStream_t st);
 int launch_fill(int32_t* p, int n, int32_t value, hipStream_t st);
 // Copies `bytes` (a multiple of 16) from pinned host memory to device memory with a kernel on
 // `st`.  For the table upload: a copy-engine transfer in the middle of a decode step costs the

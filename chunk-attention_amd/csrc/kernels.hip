@@ -25,7 +25,6 @@
 #include <type_traits>
 
 #include "kernels.h"
-#include "rotary_math.h"
 
 namespace ca {
 namespace {
@@ -221,30 +220,15 @@ struct DecodeArgs {
     int n_stream_items;   // stream items in the list
     int stream_per_wave;  // 1: every wave of a stream workgroup takes an item of its own (needs fuse_merge 0)
     int stream_nt;   // 1: private chunks are read with the non-temporal hint (see LaunchArgs)
-    // Fused decode step (STEP kAppend / kAppendRotary): the newest token of every sequence, [n_seqs, H, D].
-    // delta_tokens already counts it; its row in the pool is written by the workgroup that attends it.
+    // Fused decode step (STEP kAppend): the newest token of every sequence, [n_seqs, H, D].
+    // delta_tokens already counts it; its row in the pool is written by the merge launch.
     const half_t* k_new;
     const half_t* v_new;
-    // ... with the rotary embedding of the step's rows folded in (STEP 2): q and the new K row are
-    // rotated in registers for the sequence's position (positions[seq], or its length before the
-    // step: seq_len[seq] + delta_tokens - 1); q itself is left as it is in memory
-    const half_t* cos_sin;
-    const int64_t* positions;
-    const int32_t* seq_len;
-    int rot_dim, max_position, neox;
 };
 
-// Decode launches come in three kinds.  kForward: attention over what the pool holds.  kAppend:
-// the fused decode step (see stream_path).  kAppendRotary: the same with rotary embedding.
-constexpr int kForward = 0, kAppend = 1, kAppendRotary = 2;
-
-// The piece own = row[d0 .. d0+7] of a query or new key row of sequence `seq`, rotated.
-__device__ __forceinline__ h8 rotated_piece(const DecodeArgs& A, const half_t* __restrict__ row, int seq, int d0, h8 own) {
-    const int64_t pos = A.positions ? A.positions[seq] : int64_t(A.seq_len[seq]) + A.delta_tokens - 1;
-    const half_t* cs = A.cos_sin + rotary::clamp_pos(pos, A.max_position) * A.rot_dim;
-    return A.neox ? rotary::rotate_piece<true>(row, d0, own, cs, A.rot_dim)
-                  : rotary::rotate_piece<false>(row, d0, own, cs, A.rot_dim);
-}
+// Decode launches come in two kinds.  kForward: attention over what the pool holds.  kAppend:
+// the fused decode step (see stream_path).
+constexpr int kForward = 0, kAppend = 1;
 
 // Wave-level merge of the partial rows p0 .. p1-1 of one (sequence, head): lane l owns output
 // dims 2l, 2l+1.  Rows are taken NB at a time with all their loads in flight together and
@@ -356,11 +340,14 @@ template <> union __attribute__((aligned(16))) DecodeLds<kMixNarrow> {
 // ---------------------------------------------------------------------------------------
 // PER_WAVE: the wave works alone on its own item (all tiles, no cross-wave combine, no barrier):
 // the form for many short runs, where a workgroup per run would spend its life starting up.
-// STEP kAppend / kAppendRotary (APPEND below): the fused decode step.  The newest token of the sequence (position len - 1) has no row
-// in the pool yet: the wave whose tile holds that position takes the row from k_new / v_new
-// instead, and the 16 lanes that hold it store it into the pool.  Nobody else reads that row in
-// this launch (the last chunk of a sequence belongs to exactly one stream item), and the
-// arithmetic is that of a forward over a pool the row was appended to beforehand.
+// STEP kAppend (APPEND below): the fused decode step.  The newest token of the
+// sequence (position len - 1) has no row in the pool yet: the wave whose tile holds that position
+// takes the row from k_new / v_new instead, and the arithmetic is that of a forward over a pool
+// the row was appended to beforehand.  The row itself is written into the pool by the merge launch
+// that follows (merge_kernel's append workgroups), not here: stores scattered through a launch
+// that streams at the memory's speed cost it 9 % of its duration (256 sequences: 192 -> 209 us;
+// dirty lines leave the L2 in dribs and drabs and turn the memory bus around each time), the same
+// rows written by a launch of their own, or at the end of the merge launch, cost 1-3 us.
 template <int C, bool PER_WAVE, int STEP>
 __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, StreamPathLds& sm) {
@@ -393,8 +380,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
     const int len = it.len0 + A.delta_tokens;
 
     constexpr bool APPEND = STEP != kForward;
-    h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
-    if constexpr (STEP == kAppendRotary) qv = rotated_piece(A, q + (size_t(seq) * H + h) * D, seq, 8 * j, qv);
+    const h8 qv = *reinterpret_cast<const h8*>(q + (size_t(seq) * H + h) * D + 8 * j);
 
     float m_run = NEG_INF, l_lane = 0.f;
     float acc[8];
@@ -498,6 +484,16 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
             } else {
                 // rows past the end of the sequence hold stale data: never read into the math
                 const int vmem = (APPEND && new_here) ? vsub - 1 : vsub;  // rows that the pool holds
+                // The newest token's pieces are requested in front of the tile's own loads: loads
+                // return in order, so they are there when the tile is, at no round trip of their own.
+                uint4 kn = make_uint4(0, 0, 0, 0), vn = make_uint4(0, 0, 0, 0);
+                if constexpr (APPEND) {
+                    if (new_here) {
+                        const size_t new_off = (size_t(seq) * H + h) * D;
+                        kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
+                        vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < NL; i++) {
                     const bool ok = 4 * i + g < vmem;
@@ -507,37 +503,15 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
                 if constexpr (APPEND) {
                     if (new_here) {
                         // row vsub - 1 = 4 * i_new + g_new is the newest token: lanes (g_new, j) take
-                        // piece j of it from the caller's rows, as if it had been loaded from the
-                        // pool, and put it there
+                        // piece j of it from the caller's rows, as if it had been loaded from the pool
                         const int i_new = (vsub - 1) >> 2;
                         const bool mine = ((vsub - 1) & 3) == g;
-                        // both pieces are requested before either is used: one wait, together with
-                        // the tile's own loads, instead of a round trip each
-                        const size_t new_off = (size_t(seq) * H + h) * D;
-                        uint4 kn = *(reinterpret_cast<const uint4*>(A.k_new + new_off) + j);
-                        const uint4 vn = *(reinterpret_cast<const uint4*>(A.v_new + new_off) + j);
-                        if constexpr (STEP == kAppendRotary) {
-                            kn = __builtin_bit_cast(uint4, rotated_piece(A, A.k_new + new_off, seq, 8 * j, __builtin_bit_cast(h8, kn)));
-                        }
 #pragma unroll
                         for (int i = 0; i < NL; i++) {
                             if (i == i_new && mine) {
                                 kr[i] = kn;
                                 vr[i] = vn;
                             }
-                        }
-                        uint4* kd = const_cast<uint4*>(kp[0]);
-                        uint4* vd = const_cast<uint4*>(vp[0]);
-#pragma unroll
-                        for (int cc = 1; cc < CPT; cc++) {
-                            if (i_new / LPC == cc) {
-                                kd = const_cast<uint4*>(kp[cc]);
-                                vd = const_cast<uint4*>(vp[cc]);
-                            }
-                        }
-                        if (mine) {
-                            kd[64 * (i_new % LPC)] = kn;
-                            vd[64 * (i_new % LPC)] = vn;
                         }
                     }
                 }
@@ -686,7 +660,7 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
 //   of the 16 x 128 V block through the LDS transpose read (lds_read_tr).
 // ---------------------------------------------------------------------------------------
-template <int C, int MBT, bool ROT>
+template <int C, int MBT>
 __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, SharedPathLds<MBT>& sm) {
     constexpr int MB = MBT;  // 16-row blocks of the item
@@ -717,9 +691,6 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
-            if constexpr (ROT) {
-                if (row < it.n_rows) qreg[mb][ks] = rotated_piece(A, qp - 8 * g, it.seq_begin + row, 32 * ks + 8 * g, qreg[mb][ks]);
-            }
         }
     }
 
@@ -944,7 +915,7 @@ __device__ __forceinline__ float max_over_groups(float v) {
     return fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
 }
 
-template <int C, int MBW, bool ROT>
+template <int C, int MBW>
 __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                           int h, WidePathLds& sm) {
     static_assert(MBW == 1 || MBW == 2, "one or two 16-row blocks per wave");
@@ -977,9 +948,6 @@ __device__ __forceinline__ void wide_path(const DecodeArgs& A, const WorkItem* _
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             qreg[mb][ks] = (row < it.n_rows) ? *reinterpret_cast<const h8*>(qp + 32 * ks) : h8{ 0, 0, 0, 0, 0, 0, 0, 0 };
-            if constexpr (ROT) {
-                if (row < it.n_rows) qreg[mb][ks] = rotated_piece(A, qp - 8 * g, it.seq_begin + row, 32 * ks + 8 * g, qreg[mb][ks]);
-            }
         }
     }
     float m_run[MB];
@@ -1225,10 +1193,6 @@ struct DecodeRest {
     int32_t* counters;
     const half_t* k_new;  // fused decode step only
     const half_t* v_new;
-    const half_t* cos_sin;  // ... with rotary embedding only
-    const int64_t* positions;
-    const int32_t* seq_len;
-    int rot_dim, max_position, neox;
 };
 constexpr int kFlagFuseMerge = 1, kFlagPerWave = 2, kFlagStreamNt = 4;
 
@@ -1244,7 +1208,7 @@ __device__ __forceinline__ int xcd_unit(int b, int n) {
 }
 
 template <int C, int MIX, int STEP>
-__global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void decode_kernel(
+__global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128 || STEP != kForward) ? 2 : 3) void decode_kernel(
     const WorkItem* stream_items, const WorkItem* shared_items, const half_t* kpool, const half_t* vpool,
     const half_t* q, int n_shared_wgs, int H, int delta_tokens, int flags, float scale_log2,
     int n_stream_items, const DecodeRest rest) {
@@ -1258,9 +1222,6 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
     A.stream_per_wave = (flags & kFlagPerWave) ? 1 : 0;
     A.stream_nt = (flags & kFlagStreamNt) ? 1 : 0;
     A.k_new = rest.k_new; A.v_new = rest.v_new;
-    A.cos_sin = rest.cos_sin; A.positions = rest.positions; A.seq_len = rest.seq_len;
-    A.rot_dim = rest.rot_dim; A.max_position = rest.max_position; A.neox = rest.neox;
-    constexpr bool ROT = STEP == kAppendRotary;
     __shared__ DecodeLds<MIX> lds;
     const int bid = blockIdx.x;
     CA_STAMP(0);
@@ -1275,15 +1236,15 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
                 if (gi->flags & kItemWide) {
                     // up to 64 sequences: 16 rows per wave keep all four waves busy
                     if (gi->n_rows <= 64) {
-                        wide_path<C, 1, ROT>(A, gi, h, lds.wd);
+                        wide_path<C, 1>(A, gi, h, lds.wd);
                     } else {
-                        wide_path<C, 2, ROT>(A, gi, h, lds.wd);
+                        wide_path<C, 2>(A, gi, h, lds.wd);
                     }
                 } else {
-                    shared_path<C, 2, ROT>(A, gi, h, lds.sh);
+                    shared_path<C, 2>(A, gi, h, lds.sh);
                 }
             } else {
-                shared_path<C, 1, ROT>(A, gi, h, lds.sh);
+                shared_path<C, 1>(A, gi, h, lds.sh);
             }
         }
     } else {
@@ -1299,11 +1260,38 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128) ? 2 : 3) void dec
     CA_STAMP(3);
 }
 
-// one wave per (sequence, head)
+// What the merge launch of a fused decode step needs to write the step's new K/V rows.
+struct MergeAppend {
+    const half_t* k_new;  // [n_seqs, H, D]; null: nothing to append
+    const half_t* v_new;
+    half_t* kpool;
+    half_t* vpool;
+    const int32_t* tail_slot;
+    const int32_t* tail_fill;
+    int delta_before;         // delta_tokens before the step: the row is tail_fill + delta_before
+    int C;
+};
+
+// Workgroups [0, n_merge_wgs): one wave per (sequence, head), merging its partial rows.
+// Workgroups behind them (fused decode step only): the new token's K and V rows into the pool,
+// one thread per 16-byte piece.
 __global__ __launch_bounds__(WG) void merge_kernel(const float* __restrict__ part,
                                                    half_t* __restrict__ out,
                                                    const int32_t* __restrict__ part_ptr,
-                                                   int n_seqs, int H) {
+                                                   int n_seqs, int H, int n_merge_wgs, MergeAppend ap) {
+    if (int(blockIdx.x) >= n_merge_wgs) {
+        constexpr int pieces = D / 8;
+        const int idx = (blockIdx.x - n_merge_wgs) * WG + threadIdx.x;
+        if (idx >= n_seqs * H * pieces) return;
+        const int piece = idx % pieces, sh = idx / pieces, h = sh % H, seq = sh / H;
+        const int row = ap.tail_fill[seq] + ap.delta_before;
+        if (row < 0 || row >= ap.C) return;  // host guarantees a free row; never write outside the chunk
+        const size_t src = size_t(sh) * D + 8 * piece;
+        const size_t dst = ((size_t(ap.tail_slot[seq]) * H + h) * ap.C + row) * D + 8 * piece;
+        *reinterpret_cast<h8*>(ap.kpool + dst) = *reinterpret_cast<const h8*>(ap.k_new + src);
+        *reinterpret_cast<h8*>(ap.vpool + dst) = *reinterpret_cast<const h8*>(ap.v_new + src);
+        return;
+    }
     const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
     const int sh = blockIdx.x * NW + w;
     if (sh >= n_seqs * H) return;
@@ -1524,12 +1512,6 @@ static DecodeArgs decode_args(const LaunchArgs& a) {
     d.stream_nt = a.stream_nt ? 1 : 0;
     d.k_new = static_cast<const half_t*>(a.k_new);
     d.v_new = static_cast<const half_t*>(a.v_new);
-    d.cos_sin = a.rope ? static_cast<const half_t*>(a.rope->cos_sin_cache) : nullptr;
-    d.positions = a.rope ? a.rope->positions : nullptr;
-    d.seq_len = a.seq_len;
-    d.rot_dim = a.rope ? a.rope->rot_dim : 0;
-    d.max_position = a.rope ? a.rope->max_position : 0;
-    d.neox = a.rope && a.rope->is_neox ? 1 : 0;
     return d;
 }
 
@@ -1538,14 +1520,7 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     if (a.stream_per_wave && fuse_merge) return -1;  // waves on their own never meet at a barrier
     const bool append = a.k_new != nullptr;
     if (append && (!a.v_new || fuse_merge)) return -1;
-    if (a.rope) {
-        // rotary embedding rides on the fused step only; pieces of 8 halves must pair up
-        if (!append || !a.seq_len || !a.rope->cos_sin_cache || a.rope->max_position <= 0 || a.rope->rot_dim <= 0 ||
-            a.rope->rot_dim > D || a.rope->rot_dim % (a.rope->is_neox ? 16 : 8) != 0) {
-            return -1;
-        }
-    }
-    const int step = !append ? kForward : (a.rope ? kAppendRotary : kAppend);
+    const int step = append ? kAppend : kForward;
     const int stream_groups = a.stream_per_wave ? (n_stream_items + NW - 1) / NW : n_stream_items;
     const int64_t wgs = int64_t(n_shared_items + stream_groups) * a.H;
     if (wgs <= 0) return 0;
@@ -1555,8 +1530,7 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     d.n_stream_items = n_stream_items;
     d.stream_per_wave = a.stream_per_wave ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(wgs)), block(WG);
-    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters, d.k_new, d.v_new, d.cos_sin, d.positions,
-                           d.seq_len, d.rot_dim, d.max_position, d.neox };
+    const DecodeRest rest{ d.slots, d.out, d.part, d.part_ptr, d.counters, d.k_new, d.v_new };
     const int flags = (d.fuse_merge ? kFlagFuseMerge : 0) | (d.stream_per_wave ? kFlagPerWave : 0) |
                       (d.stream_nt ? kFlagStreamNt : 0);
     // the lightest form of the kernel that holds every path this launch takes
@@ -1568,8 +1542,7 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
 #define CA_DECODE_STEP(CS, MIX)                                           \
     do {                                                                  \
         if (step == kForward) CA_DECODE_LAUNCH(CS, MIX, kForward);        \
-        else if (step == kAppend) CA_DECODE_LAUNCH(CS, MIX, kAppend);     \
-        else CA_DECODE_LAUNCH(CS, MIX, kAppendRotary);                    \
+        else CA_DECODE_LAUNCH(CS, MIX, kAppend);                          \
     } while (0)
 #define CA_DECODE_MIX(CS)                                                 \
     do {                                                                  \
@@ -1590,11 +1563,26 @@ int launch_decode(const LaunchArgs& a, int n_shared_items, int n_stream_items, b
     return 0;
 }
 
-int launch_merge(const LaunchArgs& a, int n_seqs, hipStream_t st) {
+int launch_merge(const LaunchArgs& a, int n_seqs, bool merge, hipStream_t st) {
     if (n_seqs <= 0) return 0;
-    const int waves = n_seqs * a.H;
-    hipLaunchKernelGGL(merge_kernel, dim3((waves + NW - 1) / NW), dim3(WG), 0, st, a.part,
-                       static_cast<half_t*>(a.out), a.part_ptr, n_seqs, a.H);
+    const bool append = a.k_new != nullptr;
+    if (!merge && !append) return 0;
+    if (append && (!a.v_new || !a.tail_slot || !a.tail_fill || a.d != D)) return -1;
+    const int merge_wgs = merge ? (n_seqs * a.H + NW - 1) / NW : 0;
+    const int append_wgs = append ? (n_seqs * a.H * (D / 8) + WG - 1) / WG : 0;
+    MergeAppend ap{};
+    if (append) {
+        ap.k_new = static_cast<const half_t*>(a.k_new);
+        ap.v_new = static_cast<const half_t*>(a.v_new);
+        ap.kpool = static_cast<half_t*>(const_cast<void*>(a.kpool));
+        ap.vpool = static_cast<half_t*>(const_cast<void*>(a.vpool));
+        ap.tail_slot = a.tail_slot;
+        ap.tail_fill = a.tail_fill;
+        ap.delta_before = a.delta_tokens - 1;
+        ap.C = a.C;
+    }
+    hipLaunchKernelGGL(merge_kernel, dim3(merge_wgs + append_wgs), dim3(WG), 0, st, a.part,
+                       static_cast<half_t*>(a.out), a.part_ptr, n_seqs, a.H, merge_wgs, ap);
     CA_LAUNCH_CHECK();
     return 0;
 }

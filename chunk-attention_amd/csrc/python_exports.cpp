@@ -49,8 +49,6 @@ PYBIND11_MODULE(chunk_attn_c, m) {
            py::arg("v"), py::arg("cos_sin_cache"), py::arg("is_neox") = true, py::arg("positions") = py::none(),
            py::return_value_policy::reference)
       .def("decode_step", &Attention::decode_step, py::arg("tokens"), py::arg("q"), py::arg("k"), py::arg("v"))
-      .def("decode_step_rotary", &Attention::decode_step_rotary, py::arg("tokens"), py::arg("q"), py::arg("k"),
-           py::arg("v"), py::arg("cos_sin_cache"), py::arg("is_neox") = true, py::arg("positions") = py::none())
       .def("refresh_kernel_context", &Attention::refresh_kernel_context, py::arg("force") = false)
       .def("reserve", &Attention::reserve, py::return_value_policy::reference)
       .def("duplicate", &Attention::duplicate, py::arg("seq_idx"), py::arg("copies"))

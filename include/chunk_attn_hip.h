@@ -132,27 +132,11 @@ int ca_append_kv(ca_ctx* ctx, const void* k, const void* v, int n_seqs, void* st
  * [n_seqs, n_heads, d_head]; q attends every token including the new one.  When every sequence's
  * last chunk is streamed per sequence (always, with trees built by ca_tree_* / the Attention class
  * and tpp_threshold >= 1) no append launch is made: the workgroup that streams a sequence's last
- * chunk takes the new row from k / v and writes it into the pool on the way.  Otherwise the two
- * launches are made here.  Same preconditions as ca_append_kv (a free row in every last chunk:
+ * chunk takes the new row from k / v, and the merge launch writes the rows into the pool behind
+ * its merges.  Otherwise the two launches are made here.  Same preconditions as ca_append_kv (a free row in every last chunk:
  * reserve and refresh / ca_ctx_roll_tails first); delta_tokens is advanced by one on success. */
 int ca_decode_step(ca_ctx* ctx, const void* q, const void* k, const void* v, void* out, int n_seqs,
                    void* stream);
-
-/* ca_decode_step with the rotary embedding of the step's rows folded in: the whole decode branch
- * of the reference's attention layer (src/chunk_attn/models/llama_hf/modeling_llama.py:62,91-95:
- * rotary_embedding on the new query/key rows, append_token, forward) in one call and without a
- * launch of its own for the embedding or the append.  The results in `out` and in the pools are
- * those of  ca_rope_append_kv(positions, q, k, v, ...); ca_attention(q, out)  (same arithmetic:
- * fp32 products rounded to fp16 once), but q is only read: the workgroups rotate the rows they
- * load in registers, and the one that streams a sequence's last chunk rotates the new K row on
- * its way into the pool.  positions_dev may be NULL (position = the sequence's length before the
- * step, checked against max_position on the host).  rot_dim: a multiple of 16 (NeoX) or 8
- * (GPT-J), at most d_head.  CA_ERR_STATE when last chunks are attended chunk-first (tpp_threshold
- * 0, rows by hand) or the single-launch schedule is on: nothing was done, call ca_rope_append_kv
- * and ca_attention instead. */
-int ca_decode_step_rotary(ca_ctx* ctx, const int64_t* positions_dev, const void* q, const void* k,
-                          const void* v, const void* cos_sin_cache, int max_position, int rot_dim,
-                          int is_neox, void* out, int n_seqs, void* stream);
 
 /* Replaces rotary_embedding(positions, query, key, head_size, cos_sin_cache, is_neox)
  * (cpp/chunk_attn/pos_encoding_kernels.cu:94-139, bound as chunk_attn.ops.rotary_embedding in

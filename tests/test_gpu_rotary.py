@@ -13,7 +13,7 @@ import torch
 
 import synth
 from chunk_attn import capi
-from gpu_helpers import ATOL, RTOL, assert_close, dev, host_state, load_workload, make_attention, oracle_output, to_dev
+from gpu_helpers import ATOL, RTOL, assert_close, dev, host_state, load_workload, make_attention, to_dev
 from oracle.rotary import cos_sin_cache, rotary_embedding
 
 pytestmark = pytest.mark.gpu
@@ -124,57 +124,6 @@ def test_fused_rotate_and_append(is_neox, rot_dim):
     for slot, n_tok, _, _ in rf:       # every attended row: V identical, rotated K to the last place
         assert_one_ulp(kf[slot][:, :n_tok], kp[slot][:, :n_tok])
         assert np.array_equal(vf[slot][:, :n_tok], vp[slot][:, :n_tok])
-
-
-@pytest.mark.parametrize("is_neox,rot_dim,c,wide", [(True, 128, 32, False), (False, 128, 64, False), (True, 64, 64, False),
-                                                    (False, 40, 32, False), (True, 128, 64, True)])
-def test_decode_step_with_rotary_equals_rotary_append_then_forward(is_neox, rot_dim, c, wide):
-    """decode_step_rotary (rotary embedding and append inside the attention launch, q only read)
-    against append_token_rotary + forward on a twin cache, over decode steps that cross chunk
-    boundaries: the rotated K rows in the pool are the same bits (same arithmetic: fp32 products
-    rounded once), and so are the outputs.  `wide`: 130 sequences over one prompt, so that the
-    chunk-first items are the wide ones."""
-    H, d = 4, 128
-    rng = np.random.default_rng(15 + c + rot_dim)
-    if wide:
-        w = synth.prefix_workload("rotary-wide", 130, c, 3 * c, c // 2 + 3, n_heads=H)
-        one, _ = load_workload(w, 3)
-        two, _ = load_workload(w, 3)
-    else:
-        _, one = small_cache(H, c)
-        _, two = small_cache(H, c)
-    n = one.tree.n_seqs
-    tc = to_dev(cos_sin_cache(rot_dim, 4096))
-    for step in range(c + 2 if not wide else 4):
-        q = rng.standard_normal((n, H, d)).astype(np.float16)
-        k = rng.standard_normal((n, H, d)).astype(np.float16)
-        v = rng.standard_normal((n, H, d)).astype(np.float16)
-        toks = [5_000_000 + 100 * step + s for s in range(n)]
-        pos = None if step % 2 else to_dev(seq_lengths(two).astype(np.int64))     # both ways to give positions
-        q1, q2 = to_dev(q), to_dev(q)
-        got = one.decode_step_rotary(toks, q1, to_dev(k), to_dev(v), tc, is_neox, pos)
-        assert np.array_equal(q1.cpu().numpy(), q)              # q is only read
-        two.append_token_rotary(toks, q2, to_dev(k), to_dev(v), tc, is_neox, pos)
-        want = two.forward(q2)
-        assert torch.equal(got, want), "step %d" % step
-        assert one.ctx.delta_tokens == two.ctx.delta_tokens
-    r1, k1, v1 = host_state(one, as_float=False)
-    r2, k2, v2 = host_state(two, as_float=False)
-    assert np.array_equal(r1, r2)
-    for slot, n_tok, _, _ in r1:
-        assert np.array_equal(k1[slot][:, :n_tok].view(np.uint16), k2[slot][:, :n_tok].view(np.uint16))
-        assert np.array_equal(v1[slot][:, :n_tok].view(np.uint16), v2[slot][:, :n_tok].view(np.uint16))
-    assert_close(got, oracle_output(one, rotary_q(q, seq_lengths(one) - 1, rot_dim, is_neox)))
-    bad = to_dev(cos_sin_cache(24, 1024))
-    with pytest.raises(capi.ChunkAttnError, match="rot_dim"):
-        one.decode_step_rotary(toks, q1, to_dev(k), to_dev(v), bad)
-
-
-def rotary_q(q, positions, rot_dim, is_neox):
-    """The oracle's rotary embedding of query rows [n, H, d] at the given positions."""
-    n, H, d = q.shape
-    wq, _ = rotary_embedding(positions, q.reshape(n, H * d), q.reshape(n, H * d).copy(), d, cos_sin_cache(rot_dim, 4096), is_neox)
-    return wq.reshape(n, H, d)
 
 
 def test_fused_explicit_positions_and_errors():
