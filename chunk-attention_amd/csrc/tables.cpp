@@ -388,10 +388,23 @@ void build_plan(const ChunkRow* rows, int n_rows, int n_seqs, int chunk_size,
         const int per_wg_tokens = 512;
         const int min_chunks = std::max(4, 256 / chunk_size);
         stream_chunks = std::max(min_chunks, per_wg_tokens / chunk_size);
+        const int64_t heads = std::max(params.n_heads, 1);
         const int64_t target = int64_t(2) * params.n_cus;
-        while (stream_chunks > min_chunks &&
-               (stream_chunk_total / stream_chunks) * std::max(params.n_heads, 1) < target) {
+        while (stream_chunks > min_chunks && (stream_chunk_total / stream_chunks) * heads < target) {
             stream_chunks /= 2;
+        }
+        // Longer items where the streaming is long enough to stay balanced with them: every item
+        // but a sequence's only one leaves a partial row behind, and rows written while the launch
+        // streams cost far more than their bytes (measured with the stores switched off: 64
+        // sequences x 4096 private tokens 653 -> 608 us for 10.9 MB of rows, i.e. the memory turns
+        // its bus around for dirty lines that leave the L2 a few at a time).  Up to 2048 tokens per
+        // item as long as that leaves five fills of the device's workgroup slots (measured, 512 ->
+        // 2048 tokens: 64 x 4096 private tokens 666 -> 636 us, 64 x (1024 shared + 3072) 494 -> 488,
+        // 32 x 2560 private 207 -> 202; with fewer fills the last, partial one costs more than the
+        // rows: 64 x (3072 shared + 1024) 169 -> 173 us at 1024 tokens).
+        while (stream_chunks * 2 * chunk_size <= 2048 &&
+               (stream_chunk_total / (stream_chunks * 2)) * heads >= int64_t(10) * params.n_cus) {
+            stream_chunks *= 2;
         }
         if (stream_chunks / 2 >= min_chunks) taper_chunks = stream_chunks / 2;
     }
