@@ -560,12 +560,15 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=1, help="0-based index into the benchmark configurations (default: batch 32, 2048 shared + 512 unique, chunk 64)")
     ap.add_argument("--fraction", type=float, default=0.5, help="shared fraction for configuration 2")
+    ap.add_argument("--heads", type=int, default=32, help="number of heads (the configurations have 32; others for measurements of what depends on it)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget, 0 to skip")
     ap.add_argument("--no-paged", action="store_true", help="skip the private-copies baseline")
     ap.add_argument("--operators", action="store_true",
                     help="also time the layer operators around the attention call (rms_norm, fused_add_rms_norm and "
                          "rotary_embedding on a prefill-sized batch): outside the metric, off by default")
     ap.add_argument("--no-pybind", action="store_true", help="skip timing the forward through the pybind11 class")
+    ap.add_argument("--no-side-costs", action="store_true",
+                    help="skip the per-step side costs and the decode-step legs (profiling runs that only want the forward)")
     ap.add_argument("--no-decode-long", action="store_true", help="skip the 2048-step decode with and without re-planning (default configuration only)")
     ap.add_argument("--markers", action="store_true",
                     help="named roctx ranges around refreshes, patches, attention calls and appends (for rocprofv3 --marker-trace)")
@@ -603,7 +606,7 @@ def main() -> int:
 
     if args.markers:
         capi.set_markers(True)
-    w = synth.baseline_config(args.config, args.fraction)
+    w = synth.baseline_config(args.config, args.fraction, args.heads)
     attn = build_cache(w, torch, capi, args.seed)
     if args.seg_chunks or args.stream_chunks:
         attn.ctx.set_plan(args.seg_chunks, args.stream_chunks)
@@ -696,8 +699,9 @@ def main() -> int:
         result["forward_pybind_minus_c_abi_us"] = round(pyb_us - ms * 1e3, 2)
         result["forward_pybind_max_abs_diff"] = float((pyb_out.float() - out.float()).abs().max())
         del pyb_out
-    result["per_step_side_costs"] = side_costs(attn, w, torch, capi, args.operators)
-    result["decode_step"] = decode_step_us(w, q, torch, capi, args.seed)
+    if not args.no_side_costs:
+        result["per_step_side_costs"] = side_costs(attn, w, torch, capi, args.operators)
+        result["decode_step"] = decode_step_us(w, q, torch, capi, args.seed)
     if args.config == 1 and not args.no_decode_long:
         result["decode_long"] = decode_long(w, torch, capi, args.seed)
     if args.config == 3:

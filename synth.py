@@ -221,9 +221,15 @@ def paged_variant(w: Workload) -> Workload:
     return p
 
 
-def baseline_config(idx: int, fraction: float = 0.5) -> Workload:
+def baseline_config(idx: int, fraction: float = 0.5, n_heads: int = 32) -> Workload:
     """The five benchmark configurations (0-based index).  `fraction` is the shared-prefix
-    fraction of configuration 2 (the sharing sweep)."""
+    fraction of configuration 2 (the sharing sweep).  n_heads other than the configurations' 32
+    gives the same workload with that many heads (its name says so): for measurements of what
+    depends on the number of heads."""
+    if n_heads != 32:
+        w = baseline_config(idx, fraction)
+        return Workload("%s-h%d" % (w.name, n_heads), n_heads, w.d_head, w.chunk_size, w.sigma, seqs=w.seqs,
+                        append_steps=w.append_steps)
     if idx == 0:
         return prefix_workload("cfg1-b16-c32-1024+256", 16, 32, 1024, 256)
     if idx == 1:
