@@ -325,7 +325,7 @@ def side_costs(attn, w, torch, capi, operators=False):
     # one beam-search step on that sequence: four candidates = three tail-chunk copies and four
     # K/V rows (wall clock with a device sync; the three new sequences are removed again)
     k4 = torch.zeros((4, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
-    for rep in range(2):            # the first step loads torch's row-copy kernels: timed is the second
+    for rep in range(2):            # the first step is a warm-up: timed is the second
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         attn.append_completion(idx, [-5 - 4 * rep, -6 - 4 * rep, -7 - 4 * rep, -8 - 4 * rep], k4, k4)
@@ -333,15 +333,31 @@ def side_costs(attn, w, torch, capi, operators=False):
         beam_us = (time.perf_counter() - t0) * 1e6
         for i in (3, 2, 1):
             attn.remove_seq(idx + i)
+    # the same step eight times in a row without waiting for the device in between (candidate 0
+    # keeps extending the sequence; the 24 sequences it spawns are removed afterwards)
+    n_free = 8
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for rep in range(n_free):
+        attn.append_completion(idx, [-100 - 4 * rep, -101 - 4 * rep, -102 - 4 * rep, -103 - 4 * rep], k4, k4)
+    host_us = (time.perf_counter() - t0) * 1e6 / n_free
+    torch.cuda.synchronize()
+    beam_free_us = (time.perf_counter() - t0) * 1e6 / n_free
+    for i in range(3 * n_free, 0, -1):
+        attn.remove_seq(idx + i)
     attn.remove_seq(idx)
     attn.refresh_kernel_context()
     torch.cuda.synchronize()
     copy_bytes = 2 * 2 * T * w.n_heads * w.d_head * 2   # K and V, read and written
     base = {"table_rebuild_us": round(refresh_us, 1), "append_kv_us": round(append_us, 1),
             "add_seq_2048_tokens_us": round(add_us, 1), "add_seq_copy_GBps": round(copy_bytes / add_us / 1e3, 1),
-            "beam_step_4_candidates_us": round(beam_us, 1), "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
+            "beam_step_4_candidates_us": round(beam_us, 1), "beam_step_free_running_us": round(beam_free_us, 1), "beam_step_host_us": round(host_us, 1),
+            "scatter_kernel_2048_tokens_us": round(scatter_us, 1), "scatter_kernel_GBps": round(copy_bytes / scatter_us / 1e3, 1),
             "rotary_then_append_us": round(two_us, 1), "rotary_append_fused_us": round(fused_us, 1),
-            "chunk_rows": int(attn.ctx.plan_info().n_chunks)}
+            "chunk_rows": int(attn.ctx.plan_info().n_chunks),
+            "beam_note": "beam_step_4_candidates_us: one step from an idle device to its completion, wall clock "
+                         "with a device sync (launch + sync of an idle device alone is about 15 us); "
+                         "beam_step_free_running_us: eight steps in a row and one sync; beam_step_host_us: host time per step of those"}
     if not operators:
         return base
     # the layer's norm operators on a prefill batch of 16384 rows of H*d (128 MiB per tensor, so
