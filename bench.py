@@ -211,6 +211,29 @@ def pybind_forward_us(w, q, steps, warmup, torch, seed):
                 n_rolled += len(fresh)
             rolls += 1
     torch.cuda.synchronize()
+    # one beam-search step with four candidates through the class (three copies of the last chunk
+    # and four K/V rows in one launch): from an idle device to completion, and eight in a row
+    k4 = torch.zeros((4, w.n_heads, w.d_head), dtype=torch.float16, device="cuda:0")
+    for rep in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        attn.append_completion(0, [-5 - 4 * rep, -6 - 4 * rep, -7 - 4 * rep, -8 - 4 * rep], k4, k4)
+        torch.cuda.synchronize()
+        beam_synced = (time.perf_counter() - t0) * 1e6
+        for i in (3, 2, 1):
+            attn.remove_seq(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for rep in range(8):
+        attn.append_completion(0, [-100 - 4 * rep, -101 - 4 * rep, -102 - 4 * rep, -103 - 4 * rep], k4, k4)
+    beam_host = (time.perf_counter() - t0) * 1e6 / 8
+    torch.cuda.synchronize()
+    beam_free = (time.perf_counter() - t0) * 1e6 / 8
+    for i in range(24, 0, -1):
+        attn.remove_seq(i)
+    beam = {"synced_us": round(beam_synced, 1), "free_running_us": round(beam_free, 1), "host_us": round(beam_host, 1),
+            "note": "append_completion with four candidates through chunk_attn.Attention (pybind11): one step from an "
+                    "idle device to its completion; eight steps in a row and one sync; host time per step of those"}
     timed = max(rolls - 1, 1)
     tables = {"tree_changed_us": round(rebuild_us, 1), "tails_rolled_us": round(float(np.median(roll_t)), 1),
               "tails_rolled_max_us": round(max(roll_t), 1),
@@ -221,7 +244,7 @@ def pybind_forward_us(w, q, steps, warmup, torch, seed):
                       "chunks a successor: tables patched in place + upload (reserve_call_us is that reserve(), which "
                       "also builds one Python object per new chunk); medians over the patches timed, max = the "
                       "patch that outgrew a device buffer, if one did (buffers double)"}
-    return us, out, tables
+    return us, out, tables, beam
 
 
 def pybind_cache(w, torch, seed, extra_chunks_per_seq=1):
@@ -708,9 +731,10 @@ def main() -> int:
                                                  "one) over bytes_per_launch bytes under the same two protocols (repeated; after "
                                                  "the 1 GiB read) and over 2 GiB, HIP events around the launch")
     if not args.no_pybind:
-        pyb_us, pyb_out, pyb_tables = pybind_forward_us(w, q, args.steps, args.warmup, torch, args.seed)
+        pyb_us, pyb_out, pyb_tables, pyb_beam = pybind_forward_us(w, q, args.steps, args.warmup, torch, args.seed)
         torch.cuda.synchronize()
         result["table_refresh_pybind"] = pyb_tables
+        result["beam_step_pybind"] = pyb_beam
         result["forward_pybind_us"] = round(pyb_us, 2)
         result["forward_pybind_minus_c_abi_us"] = round(pyb_us - ms * 1e3, 2)
         result["forward_pybind_max_abs_diff"] = float((pyb_out.float() - out.float()).abs().max())
