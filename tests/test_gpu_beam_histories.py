@@ -136,3 +136,32 @@ def test_chunk_copies_and_row_writes_in_one_launch():
         assert e.value.code == -1
     with pytest.raises(capi.ChunkAttnError):
         attn.ctx.copy_chunks_put_rows([(0, 1)], k.data_ptr(), v.data_ptr(), [(0, c)], st)
+
+
+def test_more_chunk_copies_and_rows_than_one_launch_takes():
+    """70 chunk pairs and 70 rows: more than the 64 of either that one launch's argument block
+    holds, so the calls split their work over several launches; same result as tensor assignments."""
+    import torch
+    c, n = 32, 70
+    attn = make_attention(H, c, 2 * n + 4)
+    rng = torch.Generator(device="cuda").manual_seed(12)
+    kp, vp = attn.pool_views()
+    st = torch.cuda.current_stream().cuda_stream
+    kp.copy_(torch.randn(kp.shape, device="cuda", generator=rng).half())
+    vp.copy_(torch.randn(vp.shape, device="cuda", generator=rng).half())
+    k = torch.randn((n, H, 128), device="cuda", generator=rng).half()
+    v = torch.randn((n, H, 128), device="cuda", generator=rng).half()
+    pairs = [(i, n + i) for i in range(n)]
+    targets = [(n + i, (7 * i) % c) for i in range(n)]
+    want_k, want_v = kp.clone(), vp.clone()
+    for src, dst in pairs:
+        want_k[dst], want_v[dst] = want_k[src], want_v[src]
+    for i, (slot, row) in enumerate(targets):
+        want_k[slot, :, row], want_v[slot, :, row] = k[i], v[i]
+    attn.ctx.copy_chunks_put_rows(pairs, k.data_ptr(), v.data_ptr(), targets, st)
+    torch.cuda.synchronize()
+    assert torch.equal(kp, want_k) and torch.equal(vp, want_v)
+    # the copies alone, back again
+    attn.ctx.copy_chunks([(n + i, i) for i in range(n)], st)
+    torch.cuda.synchronize()
+    assert torch.equal(kp[:n], want_k[n:2 * n]) and torch.equal(vp[:n], want_v[n:2 * n])
