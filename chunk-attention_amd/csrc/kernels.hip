@@ -317,9 +317,11 @@ struct WidePathLds {
 //   kMixStream  stream items only (nothing shared, or partition 2);
 //   kMixNarrow  stream items and shared items of at most 16 sequences, none wide.
 constexpr int kMixFull = 0, kMixStream = 1, kMixNarrow = 2;
+constexpr int kNarrowLookahead = 1;  // blocks on their way in the narrow form (three workgroups per CU: 168 registers)
 template <int MIX> union DecodeLds;
 template <> union __attribute__((aligned(16))) DecodeLds<kMixFull> {
     SharedPathLds<2> sh;
+    SharedPathLds<1> sh1;
     StreamPathLds st;
     WidePathLds wd;
 };
@@ -650,8 +652,14 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 // ---------------------------------------------------------------------------------------
 // shared_path: an item = (segment of chunks, up to 32 sequences).  The segment is one token
 // stream cut into 16-token blocks; wave w takes blocks w, w+4, ... and keeps its own online-
-// softmax state, so waves never wait for each other until the final merge.  The next block's
-// K and V are requested before the current one is consumed.
+// softmax state, so waves never wait for each other until the final merge.  The K and V of the
+// next LA blocks are on their way while the current one is consumed: LA + 1 register sets used
+// in turn (the loop body is unrolled LA + 1 times, so that every set has a fixed name and no
+// block is ever copied from one set to another -- a copy would have to wait for the block it
+// copies).  Every step of the loop issues exactly one block's loads, unconditionally: past the
+// wave's last block it requests that block again (cached, never used).  With a conditional
+// request the compiler cannot know how many loads are outstanding where the paths join and waits
+// for all of them, which serialises request and use.
 //
 // Matrix-core operand layout (v_mfma_f32_16x16x*: lane l = 16*g + i):
 //   A holds row i, B holds column i, each with the k-slice of group g; D holds rows 4g..4g+3
@@ -660,10 +668,11 @@ __device__ __forceinline__ void stream_path(const DecodeArgs& A, const WorkItem*
 //   tokens), so probabilities never leave registers.  V^T comes from a wave-private LDS copy
 //   of the 16 x 128 V block through the LDS transpose read (lds_read_tr).
 // ---------------------------------------------------------------------------------------
-template <int C, int MBT>
+template <int C, int MBT, int LA>
 __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem* __restrict__ gi,
                                             int h, SharedPathLds<MBT>& sm) {
     constexpr int MB = MBT;  // 16-row blocks of the item
+    constexpr int R = LA + 1;  // register sets
     WorkItem it;
     it.seq_begin = gi->seq_begin; it.n_rows = gi->n_rows; it.slot_first = gi->slot_first;
     it.n_chunks = gi->n_chunks; it.part_row = gi->part_row; it.pos0 = gi->pos0;
@@ -705,33 +714,29 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
     }
 
     constexpr int BPC = C / 16;  // blocks per chunk
-    const int n_blocks = it.n_chunks * BPC;
-    // valid tokens of block tb (<= 0: past the end of the sequence), and its element offset
-    auto block_valid = [&](int tb) { return len - (it.pos0 + tb / BPC) * C - (tb % BPC) * 16; };
+    // blocks of the item that hold tokens of the sequences: block tb has rem - 16 * tb of them
+    const int rem = len - it.pos0 * C;
+    const int n_blocks = min(it.n_chunks * BPC, (rem + 15) >> 4);
     auto block_base = [&](int tb) {
         return ((size_t(chunk_slot(slotv, tb / BPC)) * H + h) * size_t(C) + (tb % BPC) * 16) * D;
     };
-    h8 kreg[4], knext[4];
-    uint4 vraw[4], vnext[4];
-    auto load_block = [&](int tb, h8 (&kr)[4], uint4 (&vr)[4]) {
-        const size_t base = block_base(tb);
+    h8 kq[R][4];
+    uint4 vq[R][4];
+    // requests block tb of this wave; past its last block, that one again
+    const int last_block = w + ((n_blocks - 1 - w) & ~(NW - 1));  // (only used when w < n_blocks)
+    // ka, va: the lane's addresses, handed back so that the caller can keep them alive past the
+    // block's use (see the loop)
+    auto load_block = [&](int tb, h8 (&kr)[4], uint4 (&vr)[4], const half_t*& ka, const uint4*& va) {
+        const size_t base = block_base(tb < n_blocks ? tb : last_block);
+        ka = kpool + base + size_t(i) * D + 8 * g;
+        va = reinterpret_cast<const uint4*>(vpool + base) + l;
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            kr[ks] = *reinterpret_cast<const h8*>(kpool + base + size_t(i) * D + 32 * ks + 8 * g);
-        }
+        for (int ks = 0; ks < 4; ks++) kr[ks] = *reinterpret_cast<const h8*>(ka + 32 * ks);
 #pragma unroll
-        for (int r = 0; r < 4; r++) vr[r] = *(reinterpret_cast<const uint4*>(vpool + base) + 64 * r + l);
+        for (int r = 0; r < 4; r++) vr[r] = va[64 * r];
     };
-
-    int tb = w;
-    bool have = tb < n_blocks && block_valid(tb) > 0;
-    if (have) load_block(tb, kreg, vraw);
-    while (have) {
-        const int valid = block_valid(tb);
-        const int tn = tb + NW;
-        const bool have_next = tn < n_blocks && block_valid(tn) > 0;
-        if (have_next) load_block(tn, knext, vnext);
-
+    // one block: scores, online softmax, O^T += V^T . P^T
+    auto consume = [&](const h8 (&kreg)[4], const uint4 (&vraw)[4], int valid, bool first) {
         // V block -> LDS rows (row 4r+g, dims 8i..8i+7); stale rows past the end are zeroed
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -780,7 +785,9 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
         }
 
 #ifdef CA_TIMELINE
-        if (tb == 0) CA_STAMP(1);
+        if (first) CA_STAMP(1);
+#else
+        (void)first;
 #endif
         __builtin_amdgcn_wave_barrier();
         // O^T += V^T . P^T : A = V^T (row = dim 16*db + i, k = tokens 4g..4g+3)
@@ -793,13 +800,36 @@ __device__ __forceinline__ void shared_path(const DecodeArgs& A, const WorkItem*
             }
         }
         __builtin_amdgcn_wave_barrier();
+    };
 
-        have = have_next;
-        tb = tn;
+    if (w < n_blocks) {
+        const half_t* ka;
+        const uint4* va;
+        // (the first blocks in order, oldest first: the waits inside the loop are the minimum over
+        // the ways into it, and a reordered start would make every round's first step wait longer)
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) kreg[ks] = knext[ks];
+        for (int j = 0; j < LA; j++) {
+            load_block(w + NW * j, kq[j], vq[j], ka, va);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Rounds of R steps with the loop's only exit after a round: a step past the wave's last
+        // block still requests (its last block again: cached, never used) and skips the use.  On
+        // every way to a use the same loads have been issued since the block's own, so the wait
+        // in front of it is exact; with an exit inside the round, the compiler's single-exit form
+        // of the loop would add ways that are never taken but shorten the count.
+        int tb = w;
+        do {
 #pragma unroll
-        for (int r = 0; r < 4; r++) vraw[r] = vnext[r];
+            for (int u = 0; u < R; u++) {
+                load_block(tb + NW * LA, kq[(u + LA) % R], vq[(u + LA) % R], ka, va);
+                if (tb < n_blocks) consume(kq[u], vq[u], rem - 16 * tb, tb == 0);
+                // the address registers stay in use until here: were they free once the loads are
+                // issued, the register allocator would make them the destination of the last load,
+                // and writing the next block's address would wait for that load
+                asm volatile("" ::"v"(ka), "v"(va));
+                tb += NW;
+            }
+        } while (tb < n_blocks);
     }
 
     // ---- merge the four waves ------------------------------------------------------------
@@ -1240,11 +1270,13 @@ __global__ __launch_bounds__(WG, (MIX == kMixFull || C == 128 || STEP != kForwar
                     } else {
                         wide_path<C, 2>(A, gi, h, lds.wd);
                     }
+                } else if (gi->n_rows <= 16) {
+                    shared_path<C, 1, 3>(A, gi, h, lds.sh1);
                 } else {
-                    shared_path<C, 2>(A, gi, h, lds.sh);
+                    shared_path<C, 2, 1>(A, gi, h, lds.sh);
                 }
             } else {
-                shared_path<C, 1>(A, gi, h, lds.sh);
+                shared_path<C, 1, kNarrowLookahead>(A, gi, h, lds.sh);
             }
         }
     } else {
