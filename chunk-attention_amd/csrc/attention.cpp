@@ -46,8 +46,14 @@ void Attention::init() {
     c10::DeviceGuard guard(t_options_.device());
     max_chunks_ = ChunkAllocator::max_chunks_for(memory_mb_, chunk_size_, n_heads_, d_head_, 2);
     const int64_t chunk_elems = int64_t(chunk_size_) * n_heads_ * d_head_;
-    key_storage_ = torch::empty({ chunk_elems * max_chunks_ }, t_options_);
-    value_storage_ = torch::empty({ chunk_elems * max_chunks_ }, t_options_);
+    // One allocation, the V pool right behind the K pool: how far a chunk's V rows lie from its K
+    // rows in memory decides a few percent of the streaming rate, and with two allocations that
+    // distance is whatever the driver makes of them (the reference allocates the two pools
+    // separately, chunk_allocator.cpp:43-55; the kernels only see the two base pointers).
+    const int64_t pool_elems = chunk_elems * max_chunks_;
+    torch::Tensor pools = torch::empty({ 2 * pool_elems }, t_options_);
+    key_storage_ = pools.narrow(0, 0, pool_elems);
+    value_storage_ = pools.narrow(0, pool_elems, pool_elems);
     tree_ = std::make_unique<PrefixTree>(chunk_size_, max_chunks_, share_prefix_, chunk_elems * 2 * 2);
     check(ca_ctx_create(&ctx_, n_heads_, d_head_, chunk_size_, key_storage_.data_ptr(),
                         value_storage_.data_ptr(), max_chunks_, tpp_threshold_));
